@@ -251,6 +251,7 @@ typedef struct {
 enum {
     IFA_T_EMBD = 0, IFA_T_OUT_NORM = 1, IFA_T_OUT_NORM_B = 2, IFA_T_LM_HEAD = 3,
     IFA_T_EMBD_NORM = 4,      /* layer-list models with stem 1: weight of the grouped RMS norm behind the embedding */
+    IFA_T_BIGRAM = 5,         /* layer-list models with stem 2: hashed token-pair embedding [bigram_buckets + 1][width] */
     IFA_T_ATTN_NORM = 10, IFA_T_ATTN_NORM_B = 11, IFA_T_WQ = 12, IFA_T_WK = 13, IFA_T_WV = 14, IFA_T_WO = 15,
     IFA_T_FFN_NORM = 16, IFA_T_FFN_NORM_B = 17, IFA_T_W1 = 18, IFA_T_W2 = 19, IFA_T_W3 = 20, IFA_T_MOE_GATE = 21,
     IFA_T_WQ_B = 22, IFA_T_WK_B = 23, IFA_T_WV_B = 24, IFA_T_WO_B = 25, IFA_T_W1_B = 26, IFA_T_W2_B = 27, IFA_T_W3_B = 28,
@@ -530,6 +531,41 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
                              const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,
                              void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, void *ws_f32, size_t ws_bytes, ifa_stream stream);
 
+/* The same attention over caches whose keys have been normed and rotated by ifa_qk_rope_store_f32: key rows [max_ctx][kv_heads * dim]
+ * at k_off, value rows [max_ctx][kv_heads * vdim] at v_off (they may be another layer's); window 0: every earlier position; sink != 0:
+ * exp(sink_score) joins the denominator of every head; no norm, cap or bias inside.  The tiled kernel takes heads of up to 128
+ * dimensions of any size (zero-padded to whole 32s in LDS); max_keys (0: unknown) bounds the keys a row can see, for sharing them out. */
+int ifa_attention_kv_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int vdim, float scale, int window, int keep_first, int sink,
+                         float sink_score, const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,
+                         void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, int max_keys, void *ws_f32, size_t ws_bytes,
+                         ifa_stream stream);
+/* rows of a step: per head RMS norm over dim with a weight (bf16 [dim], shared by the heads; null: no norm), then rotation of the first
+ * rot_dims dimensions, dimension i paired with i + rot_dims / 2: (u, v) -> (u cos a - v sin a, v cos a + u sin a), a = pos * freq[i]
+ * (freq_f64_dev: double [rot_dims / 2], angles formed in double).  Query heads are rewritten in place; key heads go to the K rows of
+ * the sequences' caches, the values as they are to the V rows.  k_f32 null: queries only.  dim <= 256. */
+int ifa_qk_rope_store_f32(void *q_f32, size_t ldq, int heads, const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int kv_heads, int dim, int vdim,
+                          const void *q_norm_w_bf16, const void *k_norm_w_bf16, float eps, int rot_dims, const double *freq_f64_dev, const void *seqs_dev,
+                          const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off, ifa_stream stream);
+
+/* x[t] = embed[token_t] + pair[(prev_t * mul_prev + token_t * mul_cur) mod buckets] (pair_bf16 [buckets + 1][width]; null: no second
+ * term); a sequence's first token (position 0) takes row `buckets`.  prev_t is the row before in the step, or, for the first row of a
+ * sequence that continues, the token its slot holds (one int at state_off); the sequence's last token of the step is left there. */
+int ifa_embed_pair_f32(const void *embed_bf16, int vocab, int width, const void *pair_bf16, int buckets, int mul_prev, int mul_cur, const int *tokens_dev,
+                       const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t state_off, void *x_f32,
+                       ifa_stream stream);
+/* RMS norm whose stored weight is the offset from w_offset: y (+)= x / sqrt(mean(x^2) + eps) * (w_offset + w[c]); accumulate != 0 adds into y (the
+ * residual update behind a sub-layer; y must not be x then) */
+int ifa_rmsnorm_offset_f32(const void *x_f32, size_t ldx, size_t rows, size_t cols, const void *w_bf16, float w_offset, float eps, int accumulate,
+                           void *y_f32, size_t ldy, ifa_stream stream);
+/* both norms between two sub-layers in one launch: x += m / rms(m) * (w_offset + w_after[c]), then (w_before_bf16 not null)
+ * h = x / rms(x) * (w_offset + w_before[c]) */
+int ifa_norm_add_norm_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *w_after_bf16,
+                          const void *w_before_bf16, float w_offset, float eps, void *h_f32, size_t ldh, ifa_stream stream);
+/* out[t][c] = f(gu[t][c], gu[t][cols + c]) * (row_gate ? sigmoid(row_gate[t * ldg]) : 1); kind 0 / 1 / 2 as ifa_glu_f32, kind 3:
+ * g = min(gate, limit), u = clamp(up, -limit, limit), f = g * sigmoid(1.702 g) * (u + 1) */
+int ifa_glu_ex_f32(int kind, float limit, const void *gate_up_f32, size_t ld, size_t rows, size_t cols, const void *row_gate_f32, size_t ldg,
+                   void *out_f32, size_t ldo, ifa_stream stream);
+
 /* x[t] = embed[token_t] (bf16 rows) as fp32, no position vector */
 int ifa_embed_rows_f32(const void *embed_bf16, int vocab, int width, const int *tokens_dev, size_t tokens, void *x_f32, ifa_stream stream);
 /* RMS norm in `groups` equal consecutive parts of a row: y = x / sqrt(mean_part(x^2) + eps) * w[c]; accumulate != 0: y += that (the
@@ -605,6 +641,16 @@ int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, i
                         const void *up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
                         void *y_f32, size_t ldy, int accumulate, ifa_stream stream);
 
+/* Router of the second kind: the `top` largest (logit + bias) are chosen (lowest index on ties; bias bf16 [n_all], nullable) and their
+ * weights are the softmax over the chosen values only. */
+int ifa_moe_route_top_f32(const void *logits_f32, size_t ld, size_t rows, int n_all, int top, const void *bias_bf16, int *idx_dev, void *wgt_f32,
+                          ifa_stream stream);
+/* Gated experts: E_e(h) = W_down[e] (silu(W_gate[e] h) * (W_up[e] h)); gate_up bf16 [experts][gate ff | up ff][width], down bf16
+ * [experts][width][ff]; otherwise as ifa_moe_experts_f32 (workspace: ifa_moe_workspace_bytes(rows, top, width, 3 * ff, experts)). */
+int ifa_moe_experts_gated_f32(const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int top, const void *gate_up_bf16,
+                              const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes, void *y_f32, size_t ldy,
+                              int accumulate, ifa_stream stream);
+
 /* ======================================================================== */
 /* Layer-list worker: a decoder whose layers are given one by one, each with its own sequence mixer, a 32-bit residual       */
 /* stream and bfloat16 weights (csrc/ifa_engine_layered.hip).  It is an ifa_model: finalize / kv_slots / select_kv /        */
@@ -614,13 +660,18 @@ int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, i
 /* ======================================================================== */
 enum { IFA_MIX_WINDOW_LINEAR = 1,   /* windowed softmax attention (values = keys as projected) + decayed linear attention, side by side */
        IFA_MIX_GATED_DELTA = 2,     /* gated delta rule behind short convolutions */
-       IFA_MIX_LATENT = 3 };        /* latent attention: one compressed key / value row per position, a rotated key part shared by all heads */
+       IFA_MIX_LATENT = 3,          /* latent attention: one compressed key / value row per position, a rotated key part shared by all heads */
+       IFA_MIX_ROTARY = 4 };        /* softmax attention with rotated queries / keys: grouped queries, q | k | v projections with biases, weighted
+                                     * RMS norm of q and k per head, rotation of the first a_rot_dims dimensions (pairs i, i + a_rot_dims / 2),
+                                     * values of their own size, optional sink of fixed score, optional window, keys / values of an earlier layer */
 /* wiring of a layer.  PARALLEL: h = norm1(x); x <- x + ls1 * mixer(h) + ls2 * ffn(h).  POSTNORM: the sub-layers read x itself (plus a
  * short causal convolution of x when canon_taps > 0) and the grouped RMS norm sits on their OUTPUT: x <- x + norm1(mixer(x'));
- * x <- x + norm2(ffn(x')); with depth_avg the next layer reads sum_j dwa[j] X_j over the embedding output X_0 and every layer result. */
-enum { IFA_BLOCK_PARALLEL = 0, IFA_BLOCK_POSTNORM = 1 };
+ * x <- x + norm2(ffn(x')); with depth_avg the next layer reads sum_j dwa[j] X_j over the embedding output X_0 and every layer result.
+ * SANDWICH: an RMS norm with weight (1 + w) before AND after each sub-layer: x <- x + norm1b(mixer(norm1(x))); x <- x + norm2b(ffn(norm2(x))). */
+enum { IFA_BLOCK_PARALLEL = 0, IFA_BLOCK_POSTNORM = 1, IFA_BLOCK_SANDWICH = 2 };
 enum { IFA_FFN_GATED = 0,           /* gated feed-forward (GELU tanh, biases), width `ffn` */
-       IFA_FFN_MOE = 1 };           /* mixture of experts: x_experts experts of width x_ff + x_identity identity experts, x_top per token */
+       IFA_FFN_MOE = 1,             /* mixture of experts: x_experts experts of width x_ff + x_identity identity experts, x_top per token */
+       IFA_FFN_CLAMPED = 2 };       /* width `ffn`, no biases: g = min(gate, f_limit), u = clamp(up, +-f_limit), y = down(g sigmoid(1.702 g) (u + 1)) */
 typedef struct {
     int mixer;                       /* IFA_MIX_* */
     int ffn;                         /* width of the gated feed-forward (GELU tanh, biases); 0 = none */
@@ -641,6 +692,17 @@ typedef struct {
     float m_scale, m_rot_base, m_yarn_factor, m_yarn_original, m_yarn_fast, m_yarn_slow;
     /* feed-forward kind (IFA_FFN_*) and the mixture's sizes */
     int ffn_kind, x_experts, x_identity, x_top, x_ff;
+    /* IFA_MIX_ROTARY (with a_heads, a_kv_heads, a_dim, a_scale; a_window 0 = every earlier position, a_keep_first): size of a value head,
+     * rotated dimensions (even, <= a_dim) and their base, a_sink 1: a sink of score a_sink_score joins the softmax's denominator,
+     * a_kv_layer: 0 = keys and values of its own, j + 1 = the cache rows of layer j (an earlier IFA_MIX_ROTARY layer with projections of
+     * its own and the same a_kv_heads / a_dim / a_vdim): then the layer has no k / v tensors */
+    int a_vdim, a_rot_dims, a_sink, a_kv_layer;
+    float a_rot_base, a_sink_score;
+    /* IFA_FFN_CLAMPED: the limit.  Mixture: x_gated 1 = experts down(silu(gate h) * (up h)) (IFA_LT_X_UP holds [gate rows | up rows] per
+     * expert); x_route 0 = softmax over all, choice by score + correction, weights = scores; 1 = choice by logit + bias, weights = softmax
+     * over the chosen logits; x_shared_ff > 0: a shared gated expert of that width for every row, times sigmoid(w_sg . h) */
+    float f_limit;
+    int x_gated, x_route, x_shared_ff;
 } ifa_layer_spec;
 typedef struct {
     int width, vocab, max_ctx, n_layers, device;
@@ -650,6 +712,10 @@ typedef struct {
                                       * norm (IFA_T_EMBD_NORM), grouped RMS norm before lm_head, no position vector */
     int norm_groups;                 /* parts of the grouped RMS norms (stem 1 and POSTNORM layers) */
     float logit_softcap;             /* > 0: logits <- cap * tanh(logits / cap) */
+    /* stem 2: embedding + hashed token-pair embedding (IFA_T_BIGRAM row (prev * bigram_mul_prev + token * bigram_mul_cur) mod
+     * bigram_buckets; row bigram_buckets for a sequence's first token; bigram_buckets 0: none), no position vector, RMS norm with
+     * weight (1 + w) before lm_head.  The previous token of a sequence is kept in its slot. */
+    int bigram_buckets, bigram_mul_prev, bigram_mul_cur;
 } ifa_layered_config;
 /* tensors of a layer-list model (global ones use IFA_T_EMBD / IFA_T_OUT_NORM / IFA_T_LM_HEAD with layer = -1) */
 enum {
@@ -660,7 +726,11 @@ enum {
     IFA_LT_D_G, IFA_LT_D_NORM, IFA_LT_D_O,
     IFA_LT_NORM2, IFA_LT_CANON1, IFA_LT_CANON2, IFA_LT_DWA,
     IFA_LT_M_Q, IFA_LT_M_DQ, IFA_LT_M_DQ_NORM, IFA_LT_M_UQ, IFA_LT_M_DKV, IFA_LT_M_DKV_NORM, IFA_LT_M_UK, IFA_LT_M_UV, IFA_LT_M_G, IFA_LT_M_O,
-    IFA_LT_X_ROUTER, IFA_LT_X_CORR, IFA_LT_X_UP /* [experts * ff][width] */, IFA_LT_X_DOWN /* [experts * width][ff] */, IFA_LT_END
+    IFA_LT_X_ROUTER, IFA_LT_X_CORR, IFA_LT_X_UP /* [experts * ff][width]; gated experts: [experts][gate ff | up ff][width] */, IFA_LT_X_DOWN /* [experts * width][ff] */,
+    IFA_LT_NORM1B, IFA_LT_NORM2B,                  /* SANDWICH: the norms behind the sub-layers */
+    IFA_LT_A_V, IFA_LT_A_Q_B, IFA_LT_A_K_B, IFA_LT_A_V_B, IFA_LT_A_Q_NORM, IFA_LT_A_K_NORM,      /* IFA_MIX_ROTARY (with IFA_LT_A_Q / _K / _O) */
+    IFA_LT_X_ROUTER_B, IFA_LT_X_SH_GATE, IFA_LT_X_SH_UP, IFA_LT_X_SH_DOWN, IFA_LT_X_SH_SG,
+    IFA_LT_END
 };
 int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec *layers, ifa_model **out);
 /* a tensor from HOST memory: dtype IFA_BF16 (bit patterns) or IFA_F32 (IFA_LT_L_DECAY only); shapes are checked against the specs */

@@ -180,6 +180,14 @@ SIGNATURES = {
     "ifa_moe_route_rows_f32": (_i, [_vp, _sz, _sz, _i, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "ifa_moe_workspace_bytes": (_sz, [_sz, _i, _i, _i, _i]),
     "ifa_moe_experts_f32": (_i, [_vp, _sz, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp, _sz, _i, _vp]),
+    "ifa_attention_kv_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _f, _i, _i, _i, _f, _vp, _vp, _sz, _vp, _sz, _sz, _vp, _sz, _vp, _i, _i, _i, _vp, _sz, _vp]),
+    "ifa_qk_rope_store_f32": (_i, [_vp, _sz, _i, _vp, _sz, _vp, _sz, _i, _i, _i, _vp, _vp, _f, _i, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _vp]),
+    "ifa_embed_pair_f32": (_i, [_vp, _i, _i, _vp, _i, _i, _i, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp]),
+    "ifa_rmsnorm_offset_f32": (_i, [_vp, _sz, _sz, _sz, _vp, _f, _f, _i, _vp, _sz, _vp]),
+    "ifa_norm_add_norm_f32": (_i, [_vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp, _f, _f, _vp, _sz, _vp]),
+    "ifa_glu_ex_f32": (_i, [_i, _f, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _sz, _vp]),
+    "ifa_moe_route_top_f32": (_i, [_vp, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp]),
+    "ifa_moe_experts_gated_f32": (_i, [_vp, _sz, _sz, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp, _sz, _i, _vp]),
     "ifa_model_create_layered": (_i, [_vp, _vp, C.POINTER(_vp)]),
     "ifa_model_set_tensor_host": (_i, [_vp, _i, _i, _i, _vp, _sz, _sz]),
     "ifa_model_logits_f32": (_i, [_vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_sz)]),

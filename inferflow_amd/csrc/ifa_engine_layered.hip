@@ -19,6 +19,11 @@
 // inputs in the slot), put a grouped RMS norm on each sub-layer's OUTPUT (x <- x + norm(sub(x'))), mix with latent attention (cache row
 // [latent | rotated key part] per position; single tokens take the absorbed form, prompts expanded keys / values and the tiled
 // kernel), feed forward through a mixture of experts, and hand the next layer a learned average over the depth of the stack.
+// Layers wired IFA_BLOCK_SANDWICH carry an RMS norm with weight (1 + w) before and after each sub-layer (x <- x + norm1b(mixer(norm1(x))),
+// x <- x + norm2b(ffn(norm2(x)))), mix with softmax attention over rotated queries and keys (IFA_MIX_ROTARY: K rows normed and rotated,
+// V rows of their own size; a layer may read the rows an earlier layer has written instead of projecting keys and values), and feed
+// forward through the clamped gated form or a mixture of gated experts with a router on the logits and a shared, sigmoid-gated expert.
+// Stem 2 adds a hashed token-pair embedding whose previous token lives in the slot.
 #include <algorithm>
 #include <cmath>
 #include <cstring>
@@ -47,6 +52,10 @@ struct LLayer {
     // convolution tails in the arena; rotation frequencies (double, device) and the factor on cos / sin
     size_t c_mq = 0, c_mkv = 0, c_mg = 0, o_c = 0, o_cv1 = 0, o_cv2 = 0;
     double *freq = nullptr; float rot_mult = 1.0f;
+    // SANDWICH: column of the values in the first product; the second product (what reads norm2: dense gate | up, or router | shared
+    // expert's gate logit | shared gate | shared up) with its bias vector and column offsets
+    size_t c_av = 0;
+    bf16_t *w_in2 = nullptr, *b_in2 = nullptr; size_t n_in2 = 0, c2_fg = 0, c2_router = 0, c2_sg = 0, c2_shg = 0;
     LTensor &T(int id) { return t[id - IFA_LT_NORM1]; }
     const LTensor &T(int id) const { return t[id - IFA_LT_NORM1]; }
 };
@@ -58,8 +67,8 @@ constexpr int MAX_SLOTS = 4096;
 struct LayeredNet {
     ifa_layered_config cfg;
     std::vector<LLayer> layers;
-    LTensor embd, out_norm, lm_head, embd_norm;
-    size_t arena_floats = 0;
+    LTensor embd, out_norm, lm_head, embd_norm, bigram;
+    size_t arena_floats = 0, o_prev = 0;          // (o_prev: the cell of the sequence's last token, stem 2)
     std::vector<float *> slot_ptr;       // host copy of the table (null: not allocated yet)
     float **slot_base_dev = nullptr;
     int n_slots = 1, cur_slot = 0;
@@ -108,13 +117,27 @@ bool expected_shape(const LayeredNet *n, const ifa_layer_spec &s, int li, int id
 {
     const size_t W = (size_t)n->cfg.width;
     vec = false;
-    const bool par = s.mixer == IFA_MIX_WINDOW_LINEAR, del = s.mixer == IFA_MIX_GATED_DELTA, lat = s.mixer == IFA_MIX_LATENT;
-    const bool post = s.block == IFA_BLOCK_POSTNORM, moe = has_moe(s);
+    const bool par = s.mixer == IFA_MIX_WINDOW_LINEAR, del = s.mixer == IFA_MIX_GATED_DELTA, lat = s.mixer == IFA_MIX_LATENT, rot = s.mixer == IFA_MIX_ROTARY;
+    const bool post = s.block == IFA_BLOCK_POSTNORM, sand = s.block == IFA_BLOCK_SANDWICH, moe = has_moe(s);
+    const bool own_kv = rot && s.a_kv_layer == 0, gated = s.ffn > 0 && s.ffn_kind == IFA_FFN_GATED, any_ffn = s.ffn > 0 || moe;
+    const size_t SF = (size_t)s.x_shared_ff;
     const size_t MH = (size_t)s.m_heads, MQ = MH * (size_t)(s.m_dim + s.m_rot_dim), MR = (size_t)s.m_kv_rank, XA = (size_t)(s.x_experts + s.x_identity);
     switch (id) {
     case IFA_LT_NORM1: r = 1; c = W; vec = true; return true;
-    case IFA_LT_LS1: r = 1; c = W; vec = true; return !post;
-    case IFA_LT_NORM2: r = 1; c = W; vec = true; return post && moe;
+    case IFA_LT_LS1: r = 1; c = W; vec = true; return !post && !sand;
+    case IFA_LT_NORM2: r = 1; c = W; vec = true; return (post && moe) || (sand && any_ffn);
+    case IFA_LT_NORM1B: r = 1; c = W; vec = true; return sand;
+    case IFA_LT_NORM2B: r = 1; c = W; vec = true; return sand && any_ffn;
+    case IFA_LT_A_V: r = (size_t)s.a_kv_heads * s.a_vdim; c = W; return own_kv;
+    case IFA_LT_A_Q_B: r = 1; c = (size_t)s.a_heads * s.a_dim; vec = true; return rot;
+    case IFA_LT_A_K_B: r = 1; c = (size_t)s.a_kv_heads * s.a_dim; vec = true; return own_kv;
+    case IFA_LT_A_V_B: r = 1; c = (size_t)s.a_kv_heads * s.a_vdim; vec = true; return own_kv;
+    case IFA_LT_A_Q_NORM: r = 1; c = (size_t)s.a_dim; vec = true; return rot;
+    case IFA_LT_A_K_NORM: r = 1; c = (size_t)s.a_dim; vec = true; return own_kv;
+    case IFA_LT_X_ROUTER_B: r = 1; c = XA; vec = true; return moe && s.x_route == 1;
+    case IFA_LT_X_SH_GATE: case IFA_LT_X_SH_UP: r = SF; c = W; return moe && SF > 0;
+    case IFA_LT_X_SH_DOWN: r = W; c = SF; return moe && SF > 0;
+    case IFA_LT_X_SH_SG: r = 1; c = W; vec = true; return moe && SF > 0;
     case IFA_LT_CANON1: r = W; c = (size_t)s.canon_taps; return post && s.canon_taps > 0;
     case IFA_LT_CANON2: r = W; c = (size_t)s.canon_taps; return post && s.canon_taps > 0 && moe;
     case IFA_LT_DWA: r = 1; c = (size_t)li + 2; vec = true; return post && s.depth_avg;
@@ -129,18 +152,18 @@ bool expected_shape(const LayeredNet *n, const ifa_layer_spec &s, int li, int id
     case IFA_LT_M_G: r = MH; c = W; return lat && s.m_gate;
     case IFA_LT_M_O: r = W; c = MH * (size_t)s.m_vdim; return lat;
     case IFA_LT_X_ROUTER: r = XA; c = W; return moe;
-    case IFA_LT_X_CORR: r = 1; c = XA; vec = true; return moe;
-    case IFA_LT_X_UP: r = (size_t)s.x_experts * s.x_ff; c = W; return moe && s.x_experts > 0;
+    case IFA_LT_X_CORR: r = 1; c = XA; vec = true; return moe && s.x_route == 0;
+    case IFA_LT_X_UP: r = (size_t)s.x_experts * s.x_ff * (s.x_gated ? 2 : 1); c = W; return moe && s.x_experts > 0;
     case IFA_LT_X_DOWN: r = (size_t)s.x_experts * W; c = (size_t)s.x_ff; return moe && s.x_experts > 0;
-    case IFA_LT_LS2: case IFA_LT_FFN_DOWN_B: r = 1; c = W; vec = true; return s.ffn > 0;
+    case IFA_LT_LS2: case IFA_LT_FFN_DOWN_B: r = 1; c = W; vec = true; return gated;
     case IFA_LT_FFN_GATE: case IFA_LT_FFN_UP: r = (size_t)s.ffn; c = W; return s.ffn > 0;
-    case IFA_LT_FFN_GATE_B: case IFA_LT_FFN_UP_B: r = 1; c = (size_t)s.ffn; vec = true; return s.ffn > 0;
+    case IFA_LT_FFN_GATE_B: case IFA_LT_FFN_UP_B: r = 1; c = (size_t)s.ffn; vec = true; return gated;
     case IFA_LT_FFN_DOWN: r = W; c = (size_t)s.ffn; return s.ffn > 0;
-    case IFA_LT_A_Q: r = (size_t)s.a_heads * s.a_dim; c = W; return par;
-    case IFA_LT_A_K: r = (size_t)s.a_kv_heads * s.a_dim; c = W; return par;
+    case IFA_LT_A_Q: r = (size_t)s.a_heads * s.a_dim; c = W; return par || rot;
+    case IFA_LT_A_K: r = (size_t)s.a_kv_heads * s.a_dim; c = W; return par || own_kv;
     case IFA_LT_A_REL: r = (size_t)s.a_buckets; c = (size_t)s.a_heads; return par;
     case IFA_LT_A_SINK: r = 1; c = (size_t)s.a_heads; vec = true; return par;
-    case IFA_LT_A_O: r = W; c = (size_t)s.a_heads * s.a_dim; return par;
+    case IFA_LT_A_O: r = W; c = (size_t)s.a_heads * (rot ? s.a_vdim : s.a_dim); return par || rot;
     case IFA_LT_L_Q: case IFA_LT_L_K: r = (size_t)s.l_heads * s.l_dim; c = W; return par;
     case IFA_LT_L_V: case IFA_LT_L_G: r = (size_t)s.l_heads * s.l_vdim; c = W; return par;
     case IFA_LT_L_O: r = W; c = (size_t)s.l_heads * s.l_vdim; return par;
@@ -233,7 +256,7 @@ int ensure_rows(ifa_model *m, size_t T, size_t nseq)
             IFA_HIP_CHECK(hipMalloc((void **)&n->moe_wgt, T * n->top_max * 4));
             IFA_HIP_CHECK(hipMalloc((void **)&n->moe_idx, T * n->top_max * 4));
             for (const LLayer &L : n->layers)
-                if (has_moe(L.spec)) n->moe_ws_bytes = std::max(n->moe_ws_bytes, ifa_moe_workspace_bytes(T, L.spec.x_top, (int)W, std::max(L.spec.x_ff, 1), L.spec.x_experts));
+                if (has_moe(L.spec)) n->moe_ws_bytes = std::max(n->moe_ws_bytes, ifa_moe_workspace_bytes(T, L.spec.x_top, (int)W, std::max(L.spec.x_ff, 1) * (L.spec.x_gated ? 3 : 1), L.spec.x_experts));
             IFA_HIP_CHECK(hipMalloc(&n->moe_ws, n->moe_ws_bytes));
         }
         n->scratch_rows = T;
@@ -363,6 +386,66 @@ int run_postnorm_layer(ifa_model *m, LLayer &L, size_t li, size_t T, int nseq, b
     return post_step(m, T, nseq, fused, n->m1, L.T(IFA_LT_NORM2).data, depth_of, li, ncw, ntaps, noff);
 }
 
+// one SANDWICH layer over T rows: x <- x + norm1b(attention(norm1(x))); x <- x + norm2b(ffn(norm2(x))), every norm an RMS norm with
+// weight (1 + w).  The keys enter the cache normed and rotated; a layer with a_kv_layer reads the rows that layer has written in this step.
+// The norm behind a sub-layer and the norm in front of the next one run as ONE launch (option fuse_post): h_ready says that the layer
+// before has left norm1(x) in n->h, *next_h_ready that this layer has done so for `next`.
+int run_sandwich_layer(ifa_model *m, LLayer &L, size_t T, int nseq, bool h_ready, const LLayer *next, bool *next_h_ready)
+{
+    LayeredNet *n = m->lay;
+    const ifa_layered_config &c = n->cfg;
+    const ifa_layer_spec &sp = L.spec;
+    const size_t W = (size_t)c.width, NI = L.n_in;
+    ifa_stream s = (ifa_stream)m->stream;
+    void *const *slots = (void *const *)n->slot_base_dev;
+    const bool fused = n->opt_fuse_post != 0, moe = has_moe(sp), any_ffn = sp.ffn > 0 || moe;
+    const void *next_norm = fused && next && next->spec.block == IFA_BLOCK_SANDWICH ? next->T(IFA_LT_NORM1).data : nullptr;
+    *next_h_ready = next_norm != nullptr;
+    // x += norm_after(sub); h = norm_before(x) for whatever comes next
+    auto close_sub = [&](const float *sub, const void *w_after, const void *w_before) -> int {
+        if (fused) return ifa_norm_add_norm_f32(n->x, W, T, W, sub, W, w_after, w_before, 1.0f, c.eps, n->h, W, s);
+        int r = ifa_rmsnorm_offset_f32(sub, W, T, W, w_after, 1.0f, c.eps, 1, n->x, W, s);
+        if (!r && w_before) r = ifa_rmsnorm_offset_f32(n->x, W, T, W, w_before, 1.0f, c.eps, 0, n->h, W, s);
+        return r;
+    };
+    int rc;
+    {
+        const int H = sp.a_heads, G = sp.a_kv_heads, D = sp.a_dim, DV = sp.a_vdim;
+        const size_t OV = (size_t)H * DV;
+        const bool own = sp.a_kv_layer == 0;
+        const LLayer &KV = own ? L : n->layers[(size_t)sp.a_kv_layer - 1];
+        if (!h_ready && (rc = ifa_rmsnorm_offset_f32(n->x, W, T, W, L.T(IFA_LT_NORM1).data, 1.0f, c.eps, 0, n->h, W, s))) return rc;
+        if ((rc = linear(m, L.w_in, NI, W, n->h, W, T, L.b_in, nullptr, 1.0f, 0, n->proj, NI))) return rc;
+        if ((rc = ifa_qk_rope_store_f32(n->proj + L.c_aq, NI, H, own ? n->proj + L.c_ak : nullptr, NI, own ? n->proj + L.c_av : nullptr, NI, G, D, DV,
+                                        L.T(IFA_LT_A_Q_NORM).data, own ? L.T(IFA_LT_A_K_NORM).data : nullptr, c.eps, sp.a_rot_dims, L.freq, n->seqs_dev, n->row_seq_dev, T,
+                                        slots, KV.o_k, KV.o_v, s))) return rc;
+        if ((rc = ifa_attention_kv_f32(n->proj + L.c_aq, NI, H, G, D, DV, sp.a_scale, sp.a_window, sp.a_keep_first, sp.a_sink, sp.a_sink_score, n->seqs_dev,
+                                       n->row_seq_dev, T, slots, KV.o_k, KV.o_v, n->m1, OV, n->seqs_host.data(), (int)n->seqs_host.size(), n->opt_attn_tile_min,
+                                       c.max_ctx, n->attn_ws, n->attn_ws_bytes, s))) return rc;
+        if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_A_O).data, W, OV, n->m1, OV, T, nullptr, nullptr, 1.0f, 0, n->m2, W))) return rc;
+        if ((rc = close_sub(n->m2, L.T(IFA_LT_NORM1B).data, any_ffn ? L.T(IFA_LT_NORM2).data : next_norm))) return rc;
+    }
+    if (!any_ffn) return IFA_OK;
+    const size_t N2 = L.n_in2;
+    if ((rc = linear(m, L.w_in2, N2, W, n->h, W, T, L.b_in2, nullptr, 1.0f, 0, n->proj, N2))) return rc;
+    if (!moe) {
+        const size_t F = (size_t)sp.ffn;
+        if ((rc = ifa_glu_ex_f32(3, sp.f_limit, n->proj + L.c2_fg, N2, T, F, nullptr, 0, n->m3, F, s))) return rc;
+        if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_FFN_DOWN).data, W, F, n->m3, F, T, nullptr, nullptr, 1.0f, 0, n->m2, W))) return rc;
+    } else {
+        // the router's logits (bias added by the product) are columns of the second product; the chosen experts read norm2's output
+        if ((rc = ifa_moe_route_top_f32(n->proj + L.c2_router, N2, T, sp.x_experts, sp.x_top, nullptr, n->moe_idx, n->moe_wgt, s))) return rc;
+        if ((rc = ifa_moe_experts_gated_f32(n->h, W, T, (int)W, sp.x_ff, sp.x_experts, sp.x_top, L.T(IFA_LT_X_UP).data, L.T(IFA_LT_X_DOWN).data, n->moe_idx, n->moe_wgt,
+                                            c.ops32, n->moe_ws, n->moe_ws_bytes, n->m2, W, 0, s))) return rc;
+        if (sp.x_shared_ff > 0) {      // the shared expert: its gate sigmoid(w_sg . h) multiplies the activations in front of the down-projection
+            const size_t SF = (size_t)sp.x_shared_ff;
+            if ((rc = ifa_glu_ex_f32(0, 0.0f, n->proj + L.c2_shg, N2, T, SF, n->proj + L.c2_sg, N2, n->m3, SF, s))) return rc;
+            if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_X_SH_DOWN).data, W, SF, n->m3, SF, T, nullptr, nullptr, 1.0f, 1, n->m2, W))) return rc;
+        }
+    }
+    return close_sub(n->m2, L.T(IFA_LT_NORM2B).data, next_norm);
+}
+
 // the layers of one step over T rows / nseq sequences whose tables are already on the device; leaves the residual in n->x
 int run_layers(ifa_model *m, size_t T, int nseq)
 {
@@ -376,6 +459,9 @@ int run_layers(ifa_model *m, size_t T, int nseq)
         if ((rc = ifa_embed_rows_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, T, n->h, s))) return rc;
         if ((rc = ifa_group_rmsnorm_f32(n->h, W, T, W, c.norm_groups, n->embd_norm.data, c.eps, 0, n->x, W, s))) return rc;
         if (n->any_depth_avg && (rc = ifa_group_rmsnorm_f32(n->h, W, T, W, c.norm_groups, n->embd_norm.data, c.eps, 0, n->stack, W, s))) return rc;      // plane 0
+    } else if (c.stem == 2) {
+        if ((rc = ifa_embed_pair_f32(n->embd.data, c.vocab, c.width, c.bigram_buckets > 0 ? n->bigram.data : nullptr, c.bigram_buckets, c.bigram_mul_prev, c.bigram_mul_cur,
+                                     n->tokens_dev, n->seqs_dev, n->row_seq_dev, T, slots, n->o_prev, n->x, s))) return rc;
     } else if ((rc = ifa_embed_sinpos_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, n->pos_dev, T, c.pos_base, n->x, s))) return rc;
     bool h_ready = false;
     for (size_t li = 0; li < n->layers.size(); li++) {
@@ -384,6 +470,14 @@ int run_layers(ifa_model *m, size_t T, int nseq)
         if (sp.block == IFA_BLOCK_POSTNORM) {
             bool next_ready = false;
             if ((rc = run_postnorm_layer(m, L, li, T, nseq, h_ready, li + 1 < n->layers.size() ? &n->layers[li + 1] : nullptr, &next_ready))) return rc;
+            h_ready = next_ready;
+            if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
+                IFA_HIP_CHECK(hipMemcpyAsync(n->taps + li * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
+            continue;
+        }
+        if (sp.block == IFA_BLOCK_SANDWICH) {
+            bool next_ready = false;
+            if ((rc = run_sandwich_layer(m, L, T, nseq, h_ready, li + 1 < n->layers.size() ? &n->layers[li + 1] : nullptr, &next_ready))) return rc;
             h_ready = next_ready;
             if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
                 IFA_HIP_CHECK(hipMemcpyAsync(n->taps + li * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
@@ -445,12 +539,13 @@ int run_layers(ifa_model *m, size_t T, int nseq)
     return IFA_OK;
 }
 
-// the norm in front of lm_head: layer norm without bias, or (stem 1) the grouped RMS norm
+// the norm in front of lm_head: layer norm without bias, (stem 1) the grouped RMS norm, or (stem 2) the RMS norm with weight (1 + w)
 int out_norm_rows(ifa_model *m, const float *src, size_t rows, float *dst)
 {
     LayeredNet *n = m->lay;
     const size_t W = (size_t)n->cfg.width;
     if (n->cfg.stem == 1) return ifa_group_rmsnorm_f32(src, W, rows, W, n->cfg.norm_groups, n->out_norm.data, n->cfg.eps, 0, dst, W, (ifa_stream)m->stream);
+    if (n->cfg.stem == 2) return ifa_rmsnorm_offset_f32(src, W, rows, W, n->out_norm.data, 1.0f, n->cfg.eps, 0, dst, W, (ifa_stream)m->stream);
     return ifa_layernorm_f32(1, src, W, rows, W, n->out_norm.data, n->cfg.eps, dst, W, (ifa_stream)m->stream);
 }
 
@@ -487,9 +582,9 @@ int lay_destroy(ifa_model *m)
     drop_step_graph(n);
     for (LLayer &L : n->layers) {
         for (LTensor &t : L.t) lay_free(t.data);
-        lay_free(L.w_in); lay_free(L.b_in); lay_free(L.w_conv); lay_free(L.bucket_of); lay_free(L.freq);
+        lay_free(L.w_in); lay_free(L.b_in); lay_free(L.w_conv); lay_free(L.bucket_of); lay_free(L.freq); lay_free(L.w_in2); lay_free(L.b_in2);
     }
-    lay_free(n->embd.data); lay_free(n->out_norm.data); lay_free(n->lm_head.data); lay_free(n->embd_norm.data);
+    lay_free(n->embd.data); lay_free(n->out_norm.data); lay_free(n->lm_head.data); lay_free(n->embd_norm.data); lay_free(n->bigram.data);
     lay_free(n->m4); lay_free(n->m5); lay_free(n->stack); lay_free(n->moe_wgt); lay_free(n->moe_idx); lay_free(n->moe_ws); lay_free(n->kx); lay_free(n->vx);
     for (float *p : n->slot_ptr) lay_free(p);
     lay_free(n->slot_base_dev);
@@ -523,7 +618,9 @@ int lay_finalize(ifa_model *m)
     const size_t W = (size_t)n->cfg.width;
     IFA_REQUIRE(n->embd.present() && n->out_norm.present() && n->lm_head.present(), "layer-list worker: embedding, final norm or lm_head is missing");
     IFA_REQUIRE(n->cfg.stem != 1 || n->embd_norm.present(), "layer-list worker: the norm behind the embedding is missing");
+    IFA_REQUIRE(n->cfg.stem != 2 || n->cfg.bigram_buckets <= 0 || n->bigram.present(), "layer-list worker: the token-pair embedding is missing");
     size_t off = 0;
+    if (n->cfg.stem == 2) { n->o_prev = off; off += 4; }
     n->n_in_max = n->mix_max = n->ffn_max = n->heads_max = 4;
     for (size_t li = 0; li < n->layers.size(); li++) {
         LLayer &L = n->layers[li];
@@ -573,6 +670,50 @@ int lay_finalize(ifa_model *m)
                 n->any_moe = true;
             }
             if (sp.depth_avg) n->any_depth_avg = true;
+        } else if (sp.mixer == IFA_MIX_ROTARY) {
+            const bool own = sp.a_kv_layer == 0;
+            if ((rc = cat_rows(w, b, L.T(IFA_LT_A_Q), &L.T(IFA_LT_A_Q_B), W, L.c_aq, m->stream))) return rc;
+            while (b.size() % 4) { w.resize(w.size() + W, 0); b.push_back(0); }      // (keys and values start on 16-byte borders of the product's rows)
+            if (own && ((rc = cat_rows(w, b, L.T(IFA_LT_A_K), &L.T(IFA_LT_A_K_B), W, L.c_ak, m->stream)))) return rc;
+            while (b.size() % 4) { w.resize(w.size() + W, 0); b.push_back(0); }
+            if (own && ((rc = cat_rows(w, b, L.T(IFA_LT_A_V), &L.T(IFA_LT_A_V_B), W, L.c_av, m->stream)))) return rc;
+            const int half = sp.a_rot_dims / 2;
+            std::vector<double> fr((size_t)std::max(half, 1), 0.0);
+            for (int i = 0; i < half; i++) fr[(size_t)i] = std::pow((double)sp.a_rot_base, -2.0 * i / (double)sp.a_rot_dims);
+            IFA_HIP_CHECK(hipMalloc((void **)&L.freq, fr.size() * 8));
+            IFA_HIP_CHECK(hipMemcpy(L.freq, fr.data(), fr.size() * 8, hipMemcpyHostToDevice));
+            if (own) {
+                L.o_k = off; off += align4((size_t)n->cfg.max_ctx * sp.a_kv_heads * sp.a_dim);
+                L.o_v = off; off += align4((size_t)n->cfg.max_ctx * sp.a_kv_heads * sp.a_vdim);
+            }
+            n->mix_max = std::max({n->mix_max, (size_t)sp.a_heads * sp.a_dim, (size_t)sp.a_heads * sp.a_vdim, W});
+            // the second product and the sizes of the feed-forward's buffers
+            std::vector<bf16_t> w2, b2;
+            size_t dummy;
+            if (has_moe(sp)) {
+                if ((rc = cat_rows(w2, b2, L.T(IFA_LT_X_ROUTER), sp.x_route == 1 ? &L.T(IFA_LT_X_ROUTER_B) : nullptr, W, L.c2_router, m->stream))) return rc;
+                if (sp.x_shared_ff > 0) {
+                    LTensor sg = L.T(IFA_LT_X_SH_SG); sg.rows = 1; sg.cols = W;
+                    if ((rc = cat_rows(w2, b2, sg, nullptr, W, L.c2_sg, m->stream))) return rc;
+                    while (b2.size() % 4) { w2.resize(w2.size() + W, 0); b2.push_back(0); }
+                    if ((rc = cat_rows(w2, b2, L.T(IFA_LT_X_SH_GATE), nullptr, W, L.c2_shg, m->stream)) || (rc = cat_rows(w2, b2, L.T(IFA_LT_X_SH_UP), nullptr, W, dummy, m->stream))) return rc;
+                    n->ffn_max = std::max(n->ffn_max, (size_t)sp.x_shared_ff);
+                }
+                n->top_max = std::max(n->top_max, (size_t)sp.x_top);
+                n->any_moe = true;
+            } else if (sp.ffn > 0) {
+                if ((rc = cat_rows(w2, b2, L.T(IFA_LT_FFN_GATE), nullptr, W, L.c2_fg, m->stream)) || (rc = cat_rows(w2, b2, L.T(IFA_LT_FFN_UP), nullptr, W, dummy, m->stream))) return rc;
+                n->ffn_max = std::max(n->ffn_max, (size_t)sp.ffn);
+            }
+            if (!b2.empty()) {
+                while (b2.size() % 4) { w2.resize(w2.size() + W, 0); b2.push_back(0); }
+                L.n_in2 = b2.size();
+                IFA_HIP_CHECK(hipMalloc((void **)&L.w_in2, w2.size() * 2));
+                IFA_HIP_CHECK(hipMalloc((void **)&L.b_in2, b2.size() * 2));
+                IFA_HIP_CHECK(hipMemcpy(L.w_in2, w2.data(), w2.size() * 2, hipMemcpyHostToDevice));
+                IFA_HIP_CHECK(hipMemcpy(L.b_in2, b2.data(), b2.size() * 2, hipMemcpyHostToDevice));
+                n->n_in_max = std::max(n->n_in_max, L.n_in2);
+            }
         } else if (sp.mixer == IFA_MIX_WINDOW_LINEAR) {
             if ((rc = cat_rows(w, b, L.T(IFA_LT_A_Q), nullptr, W, L.c_aq, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_A_K), nullptr, W, L.c_ak, m->stream))
                 || (rc = cat_rows(w, b, L.T(IFA_LT_L_Q), nullptr, W, L.c_lq, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_L_K), nullptr, W, L.c_lk, m->stream))
@@ -604,7 +745,7 @@ int lay_finalize(ifa_model *m)
             n->mix_max = std::max({n->mix_max, (size_t)L.conv_ch, DV});
             n->heads_max = std::max(n->heads_max, (size_t)sp.d_heads);
         }
-        if (sp.ffn > 0) {
+        if (sp.ffn > 0 && sp.block != IFA_BLOCK_SANDWICH) {
             size_t up_off;
             if ((rc = cat_rows(w, b, L.T(IFA_LT_FFN_GATE), &L.T(IFA_LT_FFN_GATE_B), W, L.c_fg, m->stream))
                 || (rc = cat_rows(w, b, L.T(IFA_LT_FFN_UP), &L.T(IFA_LT_FFN_UP_B), W, up_off, m->stream))) return rc;
@@ -620,15 +761,18 @@ int lay_finalize(ifa_model *m)
         n->n_in_max = std::max(n->n_in_max, L.n_in);
         // the separate copies of what the fused product now holds are no longer needed
         for (int id : {IFA_LT_A_Q, IFA_LT_A_K, IFA_LT_L_Q, IFA_LT_L_K, IFA_LT_L_V, IFA_LT_L_G, IFA_LT_D_Q, IFA_LT_D_K, IFA_LT_D_V, IFA_LT_D_B, IFA_LT_D_A,
-                       IFA_LT_D_G, IFA_LT_FFN_GATE, IFA_LT_FFN_UP, IFA_LT_M_Q, IFA_LT_M_DQ, IFA_LT_M_DKV, IFA_LT_M_G}) {
+                       IFA_LT_D_G, IFA_LT_FFN_GATE, IFA_LT_FFN_UP, IFA_LT_M_Q, IFA_LT_M_DQ, IFA_LT_M_DKV, IFA_LT_M_G, IFA_LT_A_V, IFA_LT_A_Q_B, IFA_LT_A_K_B,
+                       IFA_LT_A_V_B, IFA_LT_X_ROUTER_B, IFA_LT_X_SH_GATE, IFA_LT_X_SH_UP, IFA_LT_X_SH_SG}) {
             LTensor &t = L.T(id);
             if (t.data) { lay_free(t.data); t.data = nullptr; }
         }
+        if (sp.block == IFA_BLOCK_SANDWICH) { LTensor &t = L.T(IFA_LT_X_ROUTER); if (t.data) { lay_free(t.data); t.data = nullptr; } }
     }
     if (!n->attn_ws) {
         size_t per_row = 0;
         for (const LLayer &L : n->layers)
             if (L.spec.mixer == IFA_MIX_WINDOW_LINEAR) per_row = std::max(per_row, (size_t)L.spec.a_heads * 32 * ((size_t)L.spec.a_dim + 2) * 4);
+            else if (L.spec.mixer == IFA_MIX_ROTARY) per_row = std::max(per_row, (size_t)L.spec.a_heads * 32 * ((size_t)L.spec.a_vdim + 2) * 4);
             else if (L.spec.mixer == IFA_MIX_LATENT) per_row = std::max(per_row, (size_t)L.spec.m_heads * 16 * ((size_t)L.spec.m_kv_rank + 2) * 4);
         n->attn_ws_bytes = per_row * 64;
         if (n->attn_ws_bytes) IFA_HIP_CHECK(hipMalloc((void **)&n->attn_ws, n->attn_ws_bytes));
@@ -915,17 +1059,35 @@ int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec
                         "ifa_model_create_layered: layer %d: bad latent-attention sizes", l);
             IFA_REQUIRE(s.m_yarn_factor == 0.0f || (s.m_yarn_factor > 0.0f && s.m_yarn_original > 0.0f && s.m_yarn_fast > 0.0f && s.m_yarn_slow > 0.0f),
                         "ifa_model_create_layered: layer %d: bad frequency scaling", l);
+        } else if (s.mixer == IFA_MIX_ROTARY) {
+            IFA_REQUIRE(s.a_heads > 0 && s.a_kv_heads > 0 && s.a_heads % s.a_kv_heads == 0 && s.a_dim > 0 && s.a_dim <= 256 && s.a_vdim > 0 && s.a_vdim <= 1024
+                        && s.a_window >= 0 && s.a_keep_first >= 0 && s.a_rot_dims >= 0 && s.a_rot_dims <= s.a_dim && s.a_rot_dims % 2 == 0
+                        && (s.a_rot_dims == 0 || s.a_rot_base > 1.0f), "ifa_model_create_layered: layer %d: bad attention sizes", l);
+            if (s.a_kv_layer != 0) {
+                IFA_REQUIRE(s.a_kv_layer >= 1 && s.a_kv_layer <= l, "ifa_model_create_layered: layer %d reads the keys and values of layer %d, which is not an earlier layer", l, s.a_kv_layer - 1);
+                const ifa_layer_spec &o = layers[s.a_kv_layer - 1];
+                IFA_REQUIRE(o.mixer == IFA_MIX_ROTARY && o.a_kv_layer == 0 && o.a_kv_heads == s.a_kv_heads && o.a_dim == s.a_dim && o.a_vdim == s.a_vdim,
+                            "ifa_model_create_layered: layer %d: layer %d has no keys and values of its own in this layer's shape", l, s.a_kv_layer - 1);
+            }
         } else return ifa_fail(IFA_ERR_ARG, "ifa_model_create_layered: layer %d: unknown mixer %d", l, s.mixer);
-        IFA_REQUIRE((s.block == IFA_BLOCK_POSTNORM) == (s.mixer == IFA_MIX_LATENT), "ifa_model_create_layered: layer %d: mixer %d is not wired for block kind %d", l, s.mixer, s.block);
+        IFA_REQUIRE((s.block == IFA_BLOCK_POSTNORM) == (s.mixer == IFA_MIX_LATENT) && (s.block == IFA_BLOCK_SANDWICH) == (s.mixer == IFA_MIX_ROTARY),
+                    "ifa_model_create_layered: layer %d: mixer %d is not wired for block kind %d", l, s.mixer, s.block);
+        if (s.block == IFA_BLOCK_SANDWICH) {
+            if (s.ffn_kind == IFA_FFN_MOE && s.x_experts + s.x_identity > 0)
+                IFA_REQUIRE(s.ffn == 0 && s.x_identity == 0 && s.x_gated == 1 && s.x_route == 1 && s.x_experts >= 1 && s.x_experts <= 4096 && s.x_top >= 1 && s.x_top <= s.x_experts
+                            && s.x_ff > 0 && s.x_shared_ff >= 0, "ifa_model_create_layered: layer %d: bad mixture-of-experts sizes", l);
+            else IFA_REQUIRE(s.ffn == 0 || (s.ffn_kind == IFA_FFN_CLAMPED && s.f_limit > 0.0f), "ifa_model_create_layered: layer %d: this wiring takes the clamped feed-forward or a mixture", l);
+        } else
         if (s.block == IFA_BLOCK_POSTNORM) {
             IFA_REQUIRE(s.ffn == 0 && s.canon_taps >= 0 && s.canon_taps <= 64 && cfg->norm_groups >= 1 && cfg->width % cfg->norm_groups == 0,
                         "ifa_model_create_layered: layer %d: bad block sizes (norm in %d parts of width %d)", l, cfg->norm_groups, cfg->width);
             if (s.ffn_kind == IFA_FFN_MOE && s.x_experts + s.x_identity > 0)
                 IFA_REQUIRE(s.x_experts >= 0 && s.x_identity >= 0 && s.x_experts + s.x_identity <= 4096 && s.x_top >= 1 && s.x_top <= s.x_experts + s.x_identity
                             && (s.x_experts == 0 || s.x_ff > 0), "ifa_model_create_layered: layer %d: bad mixture-of-experts sizes", l);
-        } else IFA_REQUIRE(s.ffn_kind == IFA_FFN_GATED, "ifa_model_create_layered: layer %d: the mixture of experts needs the post-norm wiring", l);
+        } else IFA_REQUIRE(s.ffn_kind == IFA_FFN_GATED, "ifa_model_create_layered: layer %d: this wiring takes the gated feed-forward with biases", l);
     }
-    IFA_REQUIRE(cfg->stem == 0 || (cfg->stem == 1 && cfg->norm_groups >= 1 && cfg->width % cfg->norm_groups == 0), "ifa_model_create_layered: bad stem");
+    IFA_REQUIRE(cfg->stem == 0 || (cfg->stem == 1 && cfg->norm_groups >= 1 && cfg->width % cfg->norm_groups == 0)
+                || (cfg->stem == 2 && cfg->bigram_buckets >= 0 && cfg->bigram_buckets < (1 << 30)), "ifa_model_create_layered: bad stem");
     IFA_HIP_CHECK(hipSetDevice(cfg->device));
     ifa_model *m = new ifa_model();
     memset(&m->cfg, 0, sizeof(m->cfg));
@@ -958,6 +1120,7 @@ int ifa_model_set_tensor_host(ifa_model *m, int layer, int tensor_id, int dtype,
         else if (tensor_id == IFA_T_LM_HEAD) { t = &n->lm_head; er = V; ec = W; }
         else if (tensor_id == IFA_T_OUT_NORM) { t = &n->out_norm; er = 1; ec = W; vec = true; }
         else if (tensor_id == IFA_T_EMBD_NORM) { t = &n->embd_norm; er = 1; ec = W; vec = true; }
+        else if (tensor_id == IFA_T_BIGRAM && n->cfg.stem == 2 && n->cfg.bigram_buckets > 0) { t = &n->bigram; er = (size_t)n->cfg.bigram_buckets + 1; ec = W; }
         else return ifa_fail(IFA_ERR_ARG, "ifa_model_set_tensor_host: global tensor id %d", tensor_id);
     } else {
         IFA_REQUIRE(layer < (int)n->layers.size() && tensor_id >= IFA_LT_NORM1 && tensor_id < IFA_LT_END, "ifa_model_set_tensor_host: layer %d / tensor id %d", layer, tensor_id);

@@ -1,7 +1,9 @@
 // ifa_moe_f32.hip -- mixture of experts on 32-bit activations with bfloat16 expert matrices:
 //   router   scores = softmax(logits) over `experts` feed-forward experts followed by `identity` identity experts; the `top` largest
 //            (score + correction) are chosen, their weights are the plain scores (not renormalized)
+//            (second kind, k_moe_route_top: the `top` largest logit + bias, weights = softmax over the chosen values only)
 //   experts  y[t] (+)= sum_k wgt[t][k] * E_{idx[t][k]}(h[t]),  E_e(h) = W_down[e] act(W_up[e] h),  identity: E(h) = h
+//            (gated experts: E_e(h) = W_down[e] (silu(W_gate[e] h) * (W_up[e] h)), gate and up rows of an expert stored back to back)
 // Few rows (decode steps): every (row, choice) pair streams its expert's matrices, a wave per output (k_moe_up_rows / k_moe_down_rows).
 // Many rows: the pairs are sorted by expert (k_moe_sort: counts, offsets and tiles of 64 rows of one expert, all in one workgroup),
 // both products run grouped on the matrix cores (ifa_linear_bf16w_grouped: gather of the rows in the first, activation in its epilogue,
@@ -46,6 +48,33 @@ __global__ void __launch_bounds__(64) k_moe_route(const float *__restrict__ logi
         if (lane == 0) { idx[(size_t)t * top + k] = bi; wgt[(size_t)t * top + k] = sc[bi]; ch[bi] = -INFINITY; }
         __syncthreads();
     }
+}
+
+// one wave per row: `top` passes of argmax over logit + bias (lowest index on ties), then the softmax over the chosen values
+__global__ void __launch_bounds__(64) k_moe_route_top(const float *__restrict__ logits, size_t ld, int n_all, int top, const bf16_t *__restrict__ bias,
+                                                      int *__restrict__ idx, float *__restrict__ wgt)
+{
+    extern __shared__ float ch[];          // [n_all] choice values, [top] weights before the division
+    float *pw = ch + n_all;
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float *z = logits + (size_t)t * ld;
+    for (int e = lane; e < n_all; e += 64) ch[e] = z[e] + (bias ? bf2f(bias[e]) : 0.0f);
+    __syncthreads();
+    float first = 0.0f, sum = 0.0f;
+    for (int k = 0; k < top; k++) {
+        float best = -INFINITY; int bi = 0x7FFFFFFF;
+        for (int e = lane; e < n_all; e += 64) { const float v = ch[e]; if (v > best || (v == best && e < bi)) { best = v; bi = e; } }
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+            if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+        }
+        if (k == 0) first = best;                      // the largest of all: the softmax's reference
+        const float p = expf(best - first);
+        sum += p;
+        if (lane == 0) { idx[(size_t)t * top + k] = bi; pw[k] = p; ch[bi] = -INFINITY; }
+        __syncthreads();
+    }
+    for (int k = lane; k < top; k += 64) wgt[(size_t)t * top + k] = pw[k] / sum;
 }
 
 // Steps of a few rows: the router's product and its choice in one launch.  A workgroup per row: the waves share out the router's outputs
@@ -102,6 +131,7 @@ __global__ void __launch_bounds__(1024) k_moe_route_rows(const float *__restrict
 }
 
 // grid (ff chunks, pairs): act[p][n] = gelu(W_up[e][n] . h[t]); a wave per n at a time.  Identity pairs do nothing.
+template <bool GATED>
 __global__ void __launch_bounds__(256) k_moe_up_rows(const float *__restrict__ h, size_t ldh, int W, int F, int experts, int top, const bf16_t *__restrict__ up,
                                                      const int *__restrict__ idx, float *__restrict__ act, int vec)
 {
@@ -109,6 +139,30 @@ __global__ void __launch_bounds__(256) k_moe_up_rows(const float *__restrict__ h
     if (e >= experts) return;
     const int lane = threadIdx.x & 63, wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), nwaves = gridDim.x * (blockDim.x >> 6);
     const float *hr = h + (size_t)(p / top) * ldh;
+    if (GATED) {      // the expert's matrix holds F gate rows, then F up rows: both dots of an output side by side
+        for (int n = wave; n < F; n += nwaves) {
+            const bf16_t *wg = up + ((size_t)e * 2 * F + n) * W, *wu = wg + (size_t)F * W;
+            float ag = 0.0f, au = 0.0f;
+            if (vec) {
+#pragma unroll 2
+                for (int k = lane * 8; k < W; k += 512) {
+                    const u32x4m gv = *reinterpret_cast<const u32x4m *>(wg + k), uv = *reinterpret_cast<const u32x4m *>(wu + k);
+                    const float4 a0 = *reinterpret_cast<const float4 *>(hr + k), a1 = *reinterpret_cast<const float4 *>(hr + k + 4);
+                    const float a8[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        ag = fmaf(a8[2 * j], __uint_as_float(gv[j] << 16), ag); ag = fmaf(a8[2 * j + 1], __uint_as_float(gv[j] & 0xFFFF0000u), ag);
+                        au = fmaf(a8[2 * j], __uint_as_float(uv[j] << 16), au); au = fmaf(a8[2 * j + 1], __uint_as_float(uv[j] & 0xFFFF0000u), au);
+                    }
+                }
+            } else {
+                for (int k = lane; k < W; k += 64) { ag = fmaf(hr[k], bf2f(wg[k]), ag); au = fmaf(hr[k], bf2f(wu[k]), au); }
+            }
+            ag = wave_sum(ag); au = wave_sum(au);
+            if (lane == 0) act[(size_t)p * F + n] = silu_exact(ag) * au;
+        }
+        return;
+    }
     for (int n = wave; n < F; n += nwaves) {
         const bf16_t *w = up + ((size_t)e * F + n) * W;
         float acc = 0.0f;
@@ -263,24 +317,38 @@ int ifa_moe_route_rows_f32(const void *h_f32, size_t ldh, size_t rows, int width
     return IFA_OK;
 }
 
+int ifa_moe_route_top_f32(const void *logits_f32, size_t ld, size_t rows, int n_all, int top, const void *bias_bf16, int *idx_dev, void *wgt_f32,
+                          ifa_stream stream)
+{
+    IFA_REQUIRE(logits_f32 && idx_dev && wgt_f32, "ifa_moe_route_top_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ld >= (size_t)n_all, "ifa_moe_route_top_f32: bad shape (%d router outputs, %d chosen)", n_all, top);
+    hipLaunchKernelGGL(k_moe_route_top, dim3((unsigned)rows), dim3(64), (size_t)(n_all + top) * 4, ifa_s(stream), (const float *)logits_f32, ld, n_all, top,
+                       (const bf16_t *)bias_bf16, idx_dev, (float *)wgt_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
 size_t ifa_moe_workspace_bytes(size_t rows, int top, int width, int ff, int experts)
 {
     const size_t pairs = rows * (size_t)top;
     return al16(pairs * ff * 4) + al16(pairs * width * 4) + 3 * al16(pairs * 4) + al16(moe_tiles_max(rows, top, experts) * 12) + 16;
 }
 
-int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int identity, int top, int act,
-                        const void *up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
-                        void *y_f32, size_t ldy, int accumulate, ifa_stream stream)
+static int moe_experts(const char *who, int gated, const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int identity, int top, int act,
+                       const void *up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
+                       void *y_f32, size_t ldy, int accumulate, ifa_stream stream)
 {
-    IFA_REQUIRE(h_f32 && idx_dev && wgt_f32 && ws && y_f32 && (experts == 0 || (up_bf16 && down_bf16)), "ifa_moe_experts_f32: null pointer");
+    IFA_REQUIRE(h_f32 && idx_dev && wgt_f32 && ws && y_f32 && (experts == 0 || (up_bf16 && down_bf16)), "%s: null pointer", who);
     IFA_REQUIRE(rows > 0 && rows < 65536 && width > 0 && ff > 0 && experts >= 0 && experts <= 4096 && identity >= 0 && top >= 1 && top <= experts + identity && act == 0
-                && ldh >= (size_t)width && ldy >= (size_t)width, "ifa_moe_experts_f32: bad shape");
-    IFA_REQUIRE(ws_bytes >= ifa_moe_workspace_bytes(rows, top, width, ff, experts) && ((uintptr_t)ws & 15) == 0, "ifa_moe_experts_f32: workspace of %zu bytes, %zu needed", ws_bytes,
-                ifa_moe_workspace_bytes(rows, top, width, ff, experts));
+                && ldh >= (size_t)width && ldy >= (size_t)width, "%s: bad shape", who);
+    // gated experts: the first product leaves gate | up (2 ff values per pair) in front of the activations
+    const int ff_ws = gated ? 3 * ff : ff;
+    IFA_REQUIRE(ws_bytes >= ifa_moe_workspace_bytes(rows, top, width, ff_ws, experts) && ((uintptr_t)ws & 15) == 0, "%s: workspace of %zu bytes, %zu needed", who, ws_bytes,
+                ifa_moe_workspace_bytes(rows, top, width, ff_ws, experts));
     const size_t pairs = rows * (size_t)top;
     char *b = (char *)ws;
-    float *actb = (float *)b; b += al16(pairs * ff * 4);
+    float *actb = (float *)b; b += al16(pairs * ff_ws * 4);
+    float *gub = actb + pairs * ff;                     // [pairs][2 ff] (gated experts, many rows)
     float *yp = (float *)b; b += al16(pairs * width * 4);
     int *a_rows = (int *)b; b += al16(pairs * 4);
     int *pair_pos = (int *)b; b += al16(pairs * 4);
@@ -292,8 +360,11 @@ int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, i
     if (rows <= 8 || experts == 0) {
         const int vec_u = (width % 8 == 0 && ldh % 4 == 0 && ((uintptr_t)h_f32 & 15) == 0 && ((uintptr_t)up_bf16 & 15) == 0) ? 1 : 0;
         const int vec_d = (ff % 8 == 0 && ((uintptr_t)down_bf16 & 15) == 0) ? 1 : 0;
-        if (experts > 0)
-            hipLaunchKernelGGL(k_moe_up_rows, dim3(std::min(512u, ifa_cdiv((size_t)ff, 4)), (unsigned)pairs), dim3(256), 0, s, h, ldh, width, ff, experts, top,
+        if (experts > 0 && gated)
+            hipLaunchKernelGGL(k_moe_up_rows<true>, dim3(std::min(512u, ifa_cdiv((size_t)ff, 4)), (unsigned)pairs), dim3(256), 0, s, h, ldh, width, ff, experts, top,
+                               (const bf16_t *)up_bf16, idx_dev, actb, vec_u);
+        else if (experts > 0)
+            hipLaunchKernelGGL(k_moe_up_rows<false>, dim3(std::min(512u, ifa_cdiv((size_t)ff, 4)), (unsigned)pairs), dim3(256), 0, s, h, ldh, width, ff, experts, top,
                                (const bf16_t *)up_bf16, idx_dev, actb, vec_u);
         hipLaunchKernelGGL(k_moe_down_rows, dim3(std::min(1024u, ifa_cdiv((size_t)width, 4)), (unsigned)rows), dim3(256), 0, s, h, ldh, width, ff, experts, top,
                            (const bf16_t *)down_bf16, idx_dev, (const float *)wgt_f32, actb, accumulate ? 1 : 0, (float *)y_f32, ldy, vec_d);
@@ -301,17 +372,38 @@ int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, i
         return IFA_OK;
     }
     const size_t max_tiles = moe_tiles_max(rows, top, experts);
-    IFA_REQUIRE(max_tiles < 65536, "ifa_moe_experts_f32: %zu rows x %d choices exceed one step", rows, top);
+    IFA_REQUIRE(max_tiles < 65536, "%s: %zu rows x %d choices exceed one step", who, rows, top);
     hipLaunchKernelGGL(k_moe_sort, dim3(1), dim3(1024), (size_t)(2 * experts + 1) * 4, s, idx_dev, (const float *)wgt_f32, (int)pairs, experts, top, a_rows, pair_pos, w_sorted,
                        tile_map, n_tiles);
     IFA_LAUNCH_CHECK();
     int rc;
+    if (gated) {
+        if ((rc = ifa_linear_bf16w_grouped(up_bf16, (size_t)2 * ff, (size_t)width, experts, h_f32, ldh, a_rows, tile_map, n_tiles, max_tiles, nullptr, 0, ops32, gub, (size_t)2 * ff, stream))) return rc;
+        if ((rc = ifa_glu_f32(0, gub, (size_t)2 * ff, pairs, (size_t)ff, actb, (size_t)ff, stream))) return rc;
+    } else
     if ((rc = ifa_linear_bf16w_grouped(up_bf16, (size_t)ff, (size_t)width, experts, h_f32, ldh, a_rows, tile_map, n_tiles, max_tiles, nullptr, 1, ops32, actb, (size_t)ff, stream))) return rc;
     if ((rc = ifa_linear_bf16w_grouped(down_bf16, (size_t)width, (size_t)ff, experts, actb, (size_t)ff, nullptr, tile_map, n_tiles, max_tiles, w_sorted, 0, ops32, yp, (size_t)width, stream))) return rc;
     hipLaunchKernelGGL(k_moe_combine, dim3(ifa_cdiv((size_t)width, 256), (unsigned)rows), dim3(256), 0, s, h, ldh, width, top, pair_pos, (const float *)wgt_f32, yp,
                        accumulate ? 1 : 0, (float *)y_f32, ldy);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
+}
+
+int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int identity, int top, int act,
+                        const void *up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
+                        void *y_f32, size_t ldy, int accumulate, ifa_stream stream)
+{
+    return moe_experts("ifa_moe_experts_f32", 0, h_f32, ldh, rows, width, ff, experts, identity, top, act, up_bf16, down_bf16, idx_dev, wgt_f32, ops32, ws, ws_bytes, y_f32,
+                       ldy, accumulate, stream);
+}
+
+int ifa_moe_experts_gated_f32(const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int top, const void *gate_up_bf16,
+                              const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes, void *y_f32, size_t ldy,
+                              int accumulate, ifa_stream stream)
+{
+    IFA_REQUIRE(experts > 0, "ifa_moe_experts_gated_f32: no experts");
+    return moe_experts("ifa_moe_experts_gated_f32", 1, h_f32, ldh, rows, width, ff, experts, 0, top, 0, gate_up_bf16, down_bf16, idx_dev, wgt_f32, ops32, ws, ws_bytes,
+                       y_f32, ldy, accumulate, stream);
 }
 
 } // extern "C"

@@ -75,6 +75,77 @@ __global__ void __launch_bounds__(256) k_group_rmsnorm(const float *__restrict__
     }
 }
 
+// x[t] = embed[token_t] + pair[row_t]; row_t = (prev_t * mul_prev + token_t * mul_cur) mod buckets, or `buckets` at position 0.  The
+// workgroup of a sequence's first row is the only one that reads the token the slot holds, and it leaves the sequence's last token
+// of this step there: no other workgroup touches that cell.
+__global__ void __launch_bounds__(256) k_embed_pair(const bf16_t *__restrict__ embed, int vocab, int width, const bf16_t *__restrict__ pair, int buckets,
+                                                    int mul_prev, int mul_cur, const int *__restrict__ tokens, const SeqDesc *__restrict__ seqs,
+                                                    const int *__restrict__ row_seq, float *const *__restrict__ slot_base, size_t state_off,
+                                                    float *__restrict__ x)
+{
+    const int t = blockIdx.x;
+    const SeqDesc sd = seqs[row_seq[t]];
+    const int tok = min(max(tokens[t], 0), vocab - 1);
+    int *cell = reinterpret_cast<int *>(slot_base[sd.slot] + state_off);
+    int prow = buckets;
+    if (pair) {
+        const int pos = sd.pos0 + t - sd.row0;
+        if (pos > 0) {
+            const int prev = t > sd.row0 ? tokens[t - 1] : *cell;
+            prow = (int)(((long long)prev * mul_prev + (long long)tok * mul_cur) % (long long)buckets);
+            if (prow < 0) prow += buckets;
+        }
+    }
+    __syncthreads();      // (the read of the cell above is done in every thread before thread 0 rewrites it)
+    if (t == sd.row0 && threadIdx.x == 0) *cell = tokens[sd.row0 + sd.n - 1];
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        float v = bf2f(embed[(size_t)tok * width + c]);
+        if (pair) v += bf2f(pair[(size_t)prow * width + c]);
+        x[(size_t)t * width + c] = v;
+    }
+}
+
+// y (+)= x / sqrt(mean(x^2) + eps) * (w_off + w[c])
+__global__ void __launch_bounds__(256) k_rmsnorm_offset(const float *__restrict__ x, size_t ldx, int cols, const bf16_t *__restrict__ w, float w_off, float eps,
+                                                        int accumulate, float *__restrict__ y, size_t ldy)
+{
+    __shared__ float red[17];
+    const float *xr = x + (size_t)blockIdx.x * ldx;
+    float *yr = y + (size_t)blockIdx.x * ldy;
+    float q = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) q = fmaf(xr[c], xr[c], q);
+    const float rinv = 1.0f / sqrtf(block_sum(q, red) / (float)cols + eps);
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+        const float v = xr[c] * rinv * (w_off + (w ? bf2f(w[c]) : 0.0f));
+        yr[c] = accumulate ? yr[c] + v : v;
+    }
+}
+
+// What lies between two sub-layers of a block with norms on both sides of each, one workgroup per row:
+//   x += m / sqrt(mean(m^2) + eps) * (w_off + w_after[c]);   h = x / sqrt(mean(x^2) + eps) * (w_off + w_before[c])   (w_before null: no h)
+// The thread that updates x[c] is the one that reads it again for h.
+__global__ void __launch_bounds__(256) k_norm_add_norm(float *__restrict__ x, size_t ldx, int cols, const float *__restrict__ m, size_t ldm,
+                                                       const bf16_t *__restrict__ w_after, const bf16_t *__restrict__ w_before, float w_off, float eps,
+                                                       float *__restrict__ h, size_t ldh)
+{
+    __shared__ float red[17];
+    float *xr = x + (size_t)blockIdx.x * ldx;
+    const float *mr = m + (size_t)blockIdx.x * ldm;
+    float q = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) q = fmaf(mr[c], mr[c], q);
+    const float rinv = 1.0f / sqrtf(block_sum(q, red) / (float)cols + eps);
+    float q2 = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+        const float v = xr[c] + mr[c] * rinv * (w_off + bf2f(w_after[c]));
+        xr[c] = v;
+        q2 = fmaf(v, v, q2);
+    }
+    if (!w_before) return;
+    const float rinv2 = 1.0f / sqrtf(block_sum(q2, red) / (float)cols + eps);
+    float *hr = h + (size_t)blockIdx.x * ldh;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) hr[c] = xr[c] * rinv2 * (w_off + bf2f(w_before[c]));
+}
+
 // stack[count - 1] <- x; x <- sum_j w[j] stack[j]  (element-wise over n = rows * cols values)
 __global__ void __launch_bounds__(256) k_depth_average(float *__restrict__ x, size_t n, float *__restrict__ stack, size_t plane, int count, const bf16_t *__restrict__ w)
 {
@@ -93,15 +164,24 @@ __global__ void __launch_bounds__(256) k_softcap(float *__restrict__ x, size_t n
     if (i < n) x[i] = cap * tanhf(x[i] / cap);
 }
 
-// out[t][c] = act(gu[t][c]) * gu[t][F + c]
-__global__ void __launch_bounds__(256) k_glu_f32(int kind, const float *__restrict__ gu, size_t ld, int F, float *__restrict__ out, size_t ldo)
+// out[t][c] = act(gu[t][c]) * gu[t][F + c]  [* sigmoid(row_gate[t])];  kind 3: the clamped form g sigmoid(1.702 g) (u + 1)
+__global__ void __launch_bounds__(256) k_glu_f32(int kind, float limit, const float *__restrict__ gu, size_t ld, int F, const float *__restrict__ row_gate, size_t ldg,
+                                                 float *__restrict__ out, size_t ldo)
 {
     const float *g = gu + (size_t)blockIdx.y * ld;
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= F) return;
     const float a = g[c], u = g[F + c];
-    const float act = kind == 0 ? silu_exact(a) : (kind == 1 ? gelu_tanh_f(a) : fmaxf(a, 0.0f));
-    out[(size_t)blockIdx.y * ldo + c] = act * u;
+    float r;
+    if (kind == 3) {
+        const float gc = fminf(a, limit), uc = fminf(fmaxf(u, -limit), limit);
+        r = gc * sigmoid_f(1.702f * gc) * (uc + 1.0f);
+    } else {
+        const float act = kind == 0 ? silu_exact(a) : (kind == 1 ? gelu_tanh_f(a) : fmaxf(a, 0.0f));
+        r = act * u;
+    }
+    if (row_gate) r *= sigmoid_f(row_gate[(size_t)blockIdx.y * ldg]);
+    out[(size_t)blockIdx.y * ldo + c] = r;
 }
 
 __global__ void __launch_bounds__(1024) k_argmax_f32(const float *__restrict__ logits, int n, size_t row_stride, const int *__restrict__ excluded,
@@ -204,8 +284,43 @@ int ifa_glu_f32(int kind, const void *gate_up_f32, size_t ld, size_t rows, size_
 {
     IFA_REQUIRE(gate_up_f32 && out_f32, "ifa_glu_f32: null pointer");
     IFA_REQUIRE(kind >= 0 && kind <= 2 && rows > 0 && cols > 0 && ld >= 2 * cols && ldo >= cols, "ifa_glu_f32: bad arguments");
-    hipLaunchKernelGGL(k_glu_f32, dim3(ifa_cdiv(cols, 256), (unsigned)rows), dim3(256), 0, ifa_s(stream), kind, (const float *)gate_up_f32, ld,
-                       (int)cols, (float *)out_f32, ldo);
+    hipLaunchKernelGGL(k_glu_f32, dim3(ifa_cdiv(cols, 256), (unsigned)rows), dim3(256), 0, ifa_s(stream), kind, 0.0f, (const float *)gate_up_f32, ld,
+                       (int)cols, (const float *)nullptr, (size_t)0, (float *)out_f32, ldo);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_glu_ex_f32(int kind, float limit, const void *gate_up_f32, size_t ld, size_t rows, size_t cols, const void *row_gate_f32, size_t ldg,
+                   void *out_f32, size_t ldo, ifa_stream stream)
+{
+    IFA_REQUIRE(gate_up_f32 && out_f32, "ifa_glu_ex_f32: null pointer");
+    IFA_REQUIRE(kind >= 0 && kind <= 3 && rows > 0 && cols > 0 && ld >= 2 * cols && ldo >= cols && (kind != 3 || limit > 0.0f), "ifa_glu_ex_f32: bad arguments");
+    hipLaunchKernelGGL(k_glu_f32, dim3(ifa_cdiv(cols, 256), (unsigned)rows), dim3(256), 0, ifa_s(stream), kind, limit, (const float *)gate_up_f32, ld,
+                       (int)cols, (const float *)row_gate_f32, ldg, (float *)out_f32, ldo);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_embed_pair_f32(const void *embed_bf16, int vocab, int width, const void *pair_bf16, int buckets, int mul_prev, int mul_cur, const int *tokens_dev,
+                       const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t state_off, void *x_f32,
+                       ifa_stream stream)
+{
+    IFA_REQUIRE(embed_bf16 && tokens_dev && seqs_dev && row_seq_dev && slot_base_dev && x_f32, "ifa_embed_pair_f32: null pointer");
+    IFA_REQUIRE(vocab > 0 && width > 0 && rows > 0 && (!pair_bf16 || buckets > 0), "ifa_embed_pair_f32: bad shape");
+    hipLaunchKernelGGL(k_embed_pair, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (const bf16_t *)embed_bf16, vocab, width, (const bf16_t *)pair_bf16, buckets,
+                       mul_prev, mul_cur, tokens_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, state_off, (float *)x_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_rmsnorm_offset_f32(const void *x_f32, size_t ldx, size_t rows, size_t cols, const void *w_bf16, float w_offset, float eps, int accumulate,
+                           void *y_f32, size_t ldy, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && y_f32, "ifa_rmsnorm_offset_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && cols > 0 && ldx >= cols && ldy >= cols, "ifa_rmsnorm_offset_f32: bad arguments");
+    IFA_REQUIRE(!accumulate || x_f32 != y_f32, "ifa_rmsnorm_offset_f32: accumulating a row's norm into the row itself");
+    hipLaunchKernelGGL(k_rmsnorm_offset, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (const float *)x_f32, ldx, (int)cols, (const bf16_t *)w_bf16, w_offset, eps,
+                       accumulate ? 1 : 0, (float *)y_f32, ldy);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }
@@ -222,6 +337,17 @@ int ifa_convert_f32_f16(const void *src_f32, size_t n, void *dst_f16, ifa_stream
 {
     IFA_REQUIRE(src_f32 && dst_f16 && n > 0, "ifa_convert_f32_f16: bad arguments");
     hipLaunchKernelGGL(k_f32_to_f16, dim3(ifa_cdiv(n, 256)), dim3(256), 0, ifa_s(stream), (const float *)src_f32, n, (_Float16 *)dst_f16);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_norm_add_norm_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *w_after_bf16,
+                          const void *w_before_bf16, float w_offset, float eps, void *h_f32, size_t ldh, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && m_f32 && w_after_bf16 && (!w_before_bf16 || h_f32), "ifa_norm_add_norm_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && cols > 0 && ldx >= cols && ldm >= cols && (!w_before_bf16 || ldh >= cols) && x_f32 != m_f32, "ifa_norm_add_norm_f32: bad arguments");
+    hipLaunchKernelGGL(k_norm_add_norm, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (float *)x_f32, ldx, (int)cols, (const float *)m_f32, ldm,
+                       (const bf16_t *)w_after_bf16, (const bf16_t *)w_before_bf16, w_offset, eps, (float *)h_f32, ldh);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -15,6 +15,14 @@
 //   "latent_attention"    queries through a normed latent (q_rank), YaRN-scaled rotation when rot.scaling is given, sigmoid gate per head
 //   "latent_attention_2"  queries straight from the input, plain rotation, no gate
 // both with one cached row [kv_rank latent | rot_dim rotated key part] per position.
+//
+// Sopulorn: width / vocab / norm.eps / embedding.bigram {buckets, mul_prev, mul_cur}; the token embedding plus a hashed embedding of the
+// (previous token, token) pair; every layer has an RMS norm with weight (1 + w) before and after each sub-layer; mixer type
+//   "attention"  causal softmax attention with grouped queries, biases on q / k / v, weighted RMS norm of q and k per head, rotation of
+//                the first rot.dims dimensions of a head (pairs i, i + dims / 2), values of size vdim, one added to the softmax's
+//                denominator; "kv_from": j = the layer has no key / value tensors and reads the cache rows of layer j
+// and a feed-forward of kind "dense" (clamped: min(gate, limit) * sigmoid(1.702 .) * (clamp(up) + 1)) or "moe" (router on logits + bias,
+// softmax over the chosen, gated SiLU experts, a shared expert times sigmoid(sg . h)), or none.
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -155,6 +163,98 @@ bool ParseMuzopel(const JsonValue &root, LayeredDesc &d)
     return true;
 }
 
+// ---- Sopulorn
+bool ParseSopulorn(const JsonValue &root, LayeredDesc &d)
+{
+    memset(&d.cfg, 0, sizeof(d.cfg));
+    if (!Need(root, "width", d.cfg.width, "config") || !Need(root, "vocab", d.cfg.vocab, "config")) return false;
+    const JsonValue *norm = root.Get("norm");
+    if (!norm || !Need(*norm, "eps", d.cfg.eps, "norm")) { if (!norm) EngineSetError("config.json: norm is missing"); return false; }
+    d.cfg.stem = 2;
+    const JsonValue *emb = root.Get("embedding");
+    const JsonValue *bg = emb ? emb->Get("bigram") : nullptr;
+    if (bg && bg->type == JsonValue::Object
+        && (!Need(*bg, "buckets", d.cfg.bigram_buckets, "embedding.bigram") || !Need(*bg, "mul_prev", d.cfg.bigram_mul_prev, "embedding.bigram")
+            || !Need(*bg, "mul_cur", d.cfg.bigram_mul_cur, "embedding.bigram"))) return false;
+    const JsonValue *layers = root.Get("layers");
+    if (!layers || layers->type != JsonValue::Array || layers->arr.empty()) { EngineSetError("config.json: layers is missing or empty"); return false; }
+    for (size_t li = 0; li < layers->arr.size(); li++) {
+        const JsonValue &L = layers->arr[li];
+        ifa_layer_spec s; memset(&s, 0, sizeof(s));
+        std::string type;
+        const JsonValue *mx = L.Get("mixer");
+        if (!L.GetString("type", type) || !mx || mx->type != JsonValue::Object) { EngineSetError("config.json: layer %zu has no type / mixer", li); return false; }
+        if (type != "attention") { EngineSetError("config.json: layer %zu: unknown type \"%s\"", li, type.c_str()); return false; }
+        s.mixer = IFA_MIX_ROTARY; s.block = IFA_BLOCK_SANDWICH;
+        s.a_sink = 1; s.a_sink_score = 0.0f;          // one added to the denominator = a sink of score 0
+        if (!Need(*mx, "heads", s.a_heads, "mixer") || !Need(*mx, "kv_heads", s.a_kv_heads, "mixer") || !Need(*mx, "dim", s.a_dim, "mixer")
+            || !Need(*mx, "vdim", s.a_vdim, "mixer") || !Need(*mx, "scale", s.a_scale, "mixer")) return false;
+        const JsonValue *rot = mx->Get("rot");
+        if (rot && rot->type == JsonValue::Object && (!Need(*rot, "base", s.a_rot_base, "mixer.rot") || !Need(*rot, "dims", s.a_rot_dims, "mixer.rot"))) return false;
+        int from = -1;
+        if (mx->GetNumber("kv_from", from)) {
+            if (from < 0 || from >= (int)li) { EngineSetError("config.json: layer %zu: kv_from %d is not an earlier layer", li, from); return false; }
+            s.a_kv_layer = from + 1;
+        }
+        const JsonValue *mlp = L.Get("mlp");
+        if (mlp && mlp->type == JsonValue::Object) {
+            std::string kind;
+            mlp->GetString("kind", kind);
+            if (kind == "dense") {
+                s.ffn_kind = IFA_FFN_CLAMPED;
+                if (!Need(*mlp, "ff", s.ffn, "mlp") || !Need(*mlp, "limit", s.f_limit, "mlp")) return false;
+            } else if (kind == "moe") {
+                const JsonValue *ex = mlp->Get("expert"), *ro = mlp->Get("router"), *sh = mlp->Get("shared");
+                if (!ex || !ro) { EngineSetError("config.json: layer %zu: mlp needs expert and router", li); return false; }
+                s.ffn_kind = IFA_FFN_MOE; s.x_gated = 1; s.x_route = 1;
+                if (!Need(*ex, "ff", s.x_ff, "mlp.expert") || !Need(*ro, "experts", s.x_experts, "mlp.router") || !Need(*ro, "top", s.x_top, "mlp.router")) return false;
+                if (sh && sh->type == JsonValue::Object && !Need(*sh, "ff", s.x_shared_ff, "mlp.shared")) return false;
+            } else { EngineSetError("config.json: layer %zu: mlp.kind \"%s\" is not supported (dense, moe)", li, kind.c_str()); return false; }
+        }
+        d.layers.push_back(s);
+        d.decays.push_back(std::vector<float>());
+    }
+    d.cfg.n_layers = (int)d.layers.size();
+    return true;
+}
+
+void SopulornNames(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out)
+{
+    out.push_back({"embed", {-1, IFA_T_EMBD}});
+    if (d.cfg.bigram_buckets > 0) out.push_back({"bigram", {-1, IFA_T_BIGRAM}});
+    out.push_back({"final.norm", {-1, IFA_T_OUT_NORM}});
+    out.push_back({"head", {-1, IFA_T_LM_HEAD}});
+    for (size_t li = 0; li < d.layers.size(); li++) {
+        const ifa_layer_spec &s = d.layers[li];
+        const std::string p = "l" + std::to_string(li) + ".";
+        const int l = (int)li;
+        out.push_back({p + "norm1", {l, IFA_LT_NORM1}}); out.push_back({p + "norm1b", {l, IFA_LT_NORM1B}});
+        out.push_back({p + "mix.q", {l, IFA_LT_A_Q}}); out.push_back({p + "mix.q.b", {l, IFA_LT_A_Q_B}}); out.push_back({p + "mix.q.norm", {l, IFA_LT_A_Q_NORM}});
+        if (s.a_kv_layer == 0) {
+            out.push_back({p + "mix.k", {l, IFA_LT_A_K}}); out.push_back({p + "mix.k.b", {l, IFA_LT_A_K_B}}); out.push_back({p + "mix.k.norm", {l, IFA_LT_A_K_NORM}});
+            out.push_back({p + "mix.v", {l, IFA_LT_A_V}}); out.push_back({p + "mix.v.b", {l, IFA_LT_A_V_B}});
+        }
+        out.push_back({p + "mix.o", {l, IFA_LT_A_O}});
+        const bool moe = s.ffn_kind == IFA_FFN_MOE && s.x_experts > 0;
+        if (!moe && s.ffn <= 0) continue;
+        out.push_back({p + "norm2", {l, IFA_LT_NORM2}}); out.push_back({p + "norm2b", {l, IFA_LT_NORM2B}});
+        if (!moe) {
+            out.push_back({p + "mlp.gate", {l, IFA_LT_FFN_GATE}}); out.push_back({p + "mlp.up", {l, IFA_LT_FFN_UP}}); out.push_back({p + "mlp.down", {l, IFA_LT_FFN_DOWN}});
+            continue;
+        }
+        out.push_back({p + "mlp.router", {l, IFA_LT_X_ROUTER}}); out.push_back({p + "mlp.router.b", {l, IFA_LT_X_ROUTER_B}});
+        for (int e = 0; e < s.x_experts; e++) {      // per expert: its gate rows, then its up rows
+            out.push_back({p + "mlp.e" + std::to_string(e) + ".gate", {l, IFA_LT_X_UP}});
+            out.push_back({p + "mlp.e" + std::to_string(e) + ".up", {l, IFA_LT_X_UP}});
+        }
+        for (int e = 0; e < s.x_experts; e++) out.push_back({p + "mlp.e" + std::to_string(e) + ".down", {l, IFA_LT_X_DOWN}});
+        if (s.x_shared_ff > 0) {
+            out.push_back({p + "mlp.shared.gate", {l, IFA_LT_X_SH_GATE}}); out.push_back({p + "mlp.shared.up", {l, IFA_LT_X_SH_UP}});
+            out.push_back({p + "mlp.shared.down", {l, IFA_LT_X_SH_DOWN}}); out.push_back({p + "mlp.shared.sg", {l, IFA_LT_X_SH_SG}});
+        }
+    }
+}
+
 // tensor name -> (layer, id).  Names that share (layer, id) are parts of ONE tensor, stacked row-wise in the order given (the experts).
 void MuzopelNames(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out)
 {
@@ -236,7 +336,8 @@ struct ArchEntry {
     void (*names)(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out);
 };
 const ArchEntry kArchitectures[] = {{"Gelarax", ParseGelarax, GelaraxSizesFromTensors, GelaraxNames},
-                                    {"Muzopel", ParseMuzopel, NoSizesFromTensors, MuzopelNames}};
+                                    {"Muzopel", ParseMuzopel, NoSizesFromTensors, MuzopelNames},
+                                    {"Sopulorn", ParseSopulorn, NoSizesFromTensors, SopulornNames}};
 
 const ArchEntry *FindArch(const std::string &name)
 {
