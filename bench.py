@@ -382,17 +382,26 @@ MUZOPEL_SIZES = {   # --arch muzopel: eight layers each (three latent-attention 
 }
 
 
+SOPULORN_SIZES = {  # --arch sopulorn: eight layers each (one with the dense feed-forward, three with a mixture of experts + shared expert, twice; two layers of each four share another's keys and values)
+    "w1024": dict(width=1024, heads=8, kv_heads=2, dim=128, vdim=128, rot_dims=64, dense_ff=2816, experts=16, top=4, ff=704, shared_ff=1408),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, rot_dims=64, dense_ff=5632, experts=32, top=6, ff=1408, shared_ff=2816),
+}
+
+
 def run_arch_bench(args):
-    """--arch gelarax | muzopel: see run_gelarax_bench / the Muzopel branch below"""
+    """--arch gelarax | muzopel | sopulorn: see run_gelarax_bench / run_muzopel_bench"""
     if args.arch.lower() == "muzopel":
         return run_muzopel_bench(args)
+    if args.arch.lower() == "sopulorn":
+        return run_muzopel_bench(args, "sopulorn")
     return run_gelarax_bench(args)
 
 
-def run_muzopel_bench(args):
-    """--arch muzopel: prefill and decode throughput of Muzopel-shaped models with random bfloat16 weights (layer-list worker: latent attention, mixture
-    of experts, fp32 residual) beside the closest standard model of this framework at equal width / heads / layers / experts / expert width (Mixtral
-    wiring: full-head attention with an F16 KV cache, gated experts, F16 weights).  One JSON line; `value` = decode tokens/s of the largest size."""
+def run_muzopel_bench(args, design="muzopel"):
+    """--arch muzopel | sopulorn: prefill and decode throughput of models of that design with random bfloat16 weights (layer-list worker: latent attention
+    or rotary attention with shared key / value rows, mixture of experts, fp32 residual) beside the closest standard model of this framework at equal
+    width / heads / KV heads / layers / experts / expert width (Mixtral wiring: attention with an F16 KV cache, gated experts, F16 weights).  One JSON
+    line; `value` = decode tokens/s of the largest size."""
     import shutil
     import tempfile
     import numpy as np
@@ -411,16 +420,18 @@ def run_muzopel_bench(args):
         torch.cuda.synchronize(); t0 = time.perf_counter(); fn(); torch.cuda.synchronize()
         return time.perf_counter() - t0
 
+    sop = design == "sopulorn"
+    label = "Sopulorn" if sop else "Muzopel"
     for name in sizes:
-        sz = MUZOPEL_SIZES[name]
-        cfg = synth.muzopel_config(vocab=32000, **sz)
-        d = tempfile.mkdtemp(prefix="ifa_muzopel_", dir="/dev/shm" if os.path.isdir("/dev/shm") else None)
+        sz = (SOPULORN_SIZES if sop else MUZOPEL_SIZES)[name]
+        cfg = synth.sopulorn_config(vocab=32000, **sz) if sop else synth.muzopel_config(vocab=32000, **sz)
+        d = tempfile.mkdtemp(prefix="ifa_%s_" % design, dir="/dev/shm" if os.path.isdir("/dev/shm") else None)
         try:
-            synth.write_muzopel_dir(d, cfg, seed=1)
+            (synth.write_sopulorn_dir if sop else synth.write_muzopel_dir)(d, cfg, seed=1)
             eng = InferenceEngine.from_model_dir(d, "bfloat16", ctx, 2, False)
         finally:
             shutil.rmtree(d, ignore_errors=True)
-        shapes = synth.muzopel_tensor_shapes(cfg)
+        shapes = synth.sopulorn_tensor_shapes(cfg) if sop else synth.muzopel_tensor_shapes(cfg)
         g = {"prefill_tok_s": {}, "params": int(sum(int(np.prod(s)) for s in shapes.values()))}
         for n in lens:
             prompt = [int(t) for t in rng.integers(3, 32000, n)]
@@ -437,7 +448,7 @@ def run_muzopel_bench(args):
         g["decode_tok_s"] = steps / wall; g["decode_ms_per_step"] = wall * 1e3 / steps; g["decode_context"] = "%d..%d" % (lens[-1] + warmup, lens[-1] + warmup + steps)
         eng.close()
         # the closest standard model: same width, heads, layer count, experts, choices per token and expert width, F16 weights
-        synth.SHAPES["cmp_" + name] = dict(dim=sz["width"], layers=8, heads=sz["heads"], kv_heads=sz["heads"], head_dim=128, ffn=sz["ff"], vocab=32000,
+        synth.SHAPES["cmp_" + name] = dict(dim=sz["width"], layers=8, heads=sz["heads"], kv_heads=sz.get("kv_heads", sz["heads"]), head_dim=128, ffn=sz["ff"], vocab=32000,
                                            experts=sz["experts"], moe_top_k=sz["top"])
         wk, _, _ = synth.build("cmp_" + name, dt.F16, dt.F16, ctx, quant_threshold=1 << 62)
         c = {"prefill_tok_s": {}}
@@ -451,12 +462,12 @@ def run_muzopel_bench(args):
         wall = timed(lambda: wk.decode(nxt, lens[-1] + warmup, steps))
         c["decode_tok_s"] = steps / wall; c["decode_ms_per_step"] = wall * 1e3 / steps
         del wk
-        rows.append({"size": name, "layers": 8, **sz, "muzopel": g, "closest_standard_model": c})
-    last = rows[-1]["muzopel"]
-    print(json.dumps({"metric": "decode tokens/sec, Muzopel-shaped model (%s), batch=1 greedy" % sizes[-1], "value": last["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1,
+        rows.append({"size": name, "layers": 8, **sz, design: g, "closest_standard_model": c})
+    last = rows[-1][design]
+    print(json.dumps({"metric": "decode tokens/sec, %s-shaped model (%s), batch=1 greedy" % (label, sizes[-1]), "value": last["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1,
                       "steps": steps, "warmup": warmup, "ms_per_step": last["decode_ms_per_step"], "higher_is_better": True, "scaling": "strong", "vs_baseline": None,
                       "dtype": "bf16 weights and matrix-product operands, f32 accumulation, residual, scores and cache", "data": "synthetic",
-                      "config": {"model": "Muzopel-shaped, random weights", "global_batch": 1, "seq_len": lens[-1], "parallelism": "single"}, "sizes": rows}))
+                      "config": {"model": "%s-shaped, random weights" % label, "global_batch": 1, "seq_len": lens[-1], "parallelism": "single"}, "sizes": rows}))
 
 
 def run_gelarax_bench(args):
@@ -548,13 +559,13 @@ def main():
                     "a functional check of the N > 1 step logic on a one-GPU box, not a scaling number")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="CPU baseline sample size (0 = auto)")
-    ap.add_argument("--arch", default="", help="'gelarax' or 'muzopel': instead of the headline workload, prefill / decode rates of models of that design beside the "
+    ap.add_argument("--arch", default="", help="'gelarax', 'muzopel' or 'sopulorn': instead of the headline workload, prefill / decode rates of models of that design beside the "
                     "closest standard model at equal size (one GPU; --prefill-lens, --steps, --warmup apply)")
     ap.add_argument("--arch-sizes", default="w1024,w2048")
     args = ap.parse_args()
     if args.arch:
-        if args.arch.lower() not in ("gelarax", "muzopel"):
-            raise SystemExit("unknown --arch %s (gelarax, muzopel)" % args.arch)
+        if args.arch.lower() not in ("gelarax", "muzopel", "sopulorn"):
+            raise SystemExit("unknown --arch %s (gelarax, muzopel, sopulorn)" % args.arch)
         if args.gpus > 1 or int(os.environ.get("WORLD_SIZE", "1")) > 1:
             raise SystemExit("--arch runs on one GPU")
         return run_arch_bench(args)

@@ -209,6 +209,55 @@ def muzopel_tensor_shapes(cfg):
     return s
 
 
+def sopulorn_config(width=2048, blocks=2, vocab=32000, heads=16, kv_heads=4, dim=128, vdim=128, rot_dims=64, dense_ff=5632, experts=32, top=6, ff=1408, shared_ff=2816):
+    """`blocks` x (one layer with the clamped dense feed-forward, three with a mixture of gated experts + a shared expert; the last two of each
+    block read the keys and values of the block's second layer)"""
+    def layer(mlp, kv_from=None):
+        mx = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": float(dim ** -0.5), "rot": {"base": 10000.0, "dims": rot_dims}}
+        if kv_from is not None:
+            mx["kv_from"] = kv_from
+        return {"type": "attention", "mixer": mx, "mlp": mlp}
+    moe = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}, "shared": {"ff": shared_ff}}
+    layers = []
+    for b in range(blocks):
+        layers += [layer({"kind": "dense", "ff": dense_ff, "limit": 7.0}), layer(moe), layer(moe, 4 * b + 1), layer(moe, 4 * b + 1)]
+    return {"architecture": "Sopulorn", "width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31337, "mul_cur": 7919}},
+            "layers": layers}
+
+
+def sopulorn_tensor_shapes(cfg):
+    W_, V = cfg["width"], cfg["vocab"]
+    s = {"embed": (V, W_), "final.norm": (W_,), "head": (V, W_)}
+    bg = (cfg.get("embedding") or {}).get("bigram")
+    if bg:
+        s["bigram"] = (bg["buckets"] + 1, W_)
+    for li, L in enumerate(cfg["layers"]):
+        p, m = "l%d." % li, L["mixer"]
+        H, G, D, DV = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        s.update({p + "norm1": (W_,), p + "norm1b": (W_,), p + "mix.q": (H * D, W_), p + "mix.q.b": (H * D,), p + "mix.q.norm": (D,), p + "mix.o": (W_, H * DV)})
+        if m.get("kv_from") is None:
+            s.update({p + "mix.k": (G * D, W_), p + "mix.k.b": (G * D,), p + "mix.k.norm": (D,), p + "mix.v": (G * DV, W_), p + "mix.v.b": (G * DV,)})
+        mlp = L.get("mlp")
+        if not mlp:
+            continue
+        s.update({p + "norm2": (W_,), p + "norm2b": (W_,)})
+        if mlp["kind"] == "dense":
+            s.update({p + "mlp.gate": (mlp["ff"], W_), p + "mlp.up": (mlp["ff"], W_), p + "mlp.down": (W_, mlp["ff"])})
+            continue
+        E, F = mlp["router"]["experts"], mlp["expert"]["ff"]
+        s.update({p + "mlp.router": (E, W_), p + "mlp.router.b": (E,)})
+        for e in range(E):
+            s.update({p + "mlp.e%d.gate" % e: (F, W_), p + "mlp.e%d.up" % e: (F, W_), p + "mlp.e%d.down" % e: (W_, F)})
+        if mlp.get("shared"):
+            S = mlp["shared"]["ff"]
+            s.update({p + "mlp.shared.gate": (S, W_), p + "mlp.shared.up": (S, W_), p + "mlp.shared.down": (W_, S), p + "mlp.shared.sg": (1, W_)})
+    return s
+
+
+def write_sopulorn_dir(path, cfg, seed=0):
+    return write_gelarax_dir(path, cfg, seed, sopulorn_tensor_shapes(cfg))
+
+
 def write_muzopel_dir(path, cfg, seed=0):
     return write_gelarax_dir(path, cfg, seed, muzopel_tensor_shapes(cfg))
 
@@ -236,7 +285,9 @@ def write_gelarax_dir(path, cfg, seed=0, shapes=None):
         f.write(struct.pack("<Q", len(hj))); f.write(hj)
         for name, shape in shapes.items():
             leaf = name.split(".")[-1]
-            if len(shape) == 1 and leaf in ("norm1", "norm2", "norm", "ls1", "ls2"):
+            if cfg.get("architecture") == "Sopulorn" and len(shape) == 1 and (leaf in ("norm1", "norm2", "norm1b", "norm2b") or name == "final.norm"):
+                a = 0.05 * rng.standard_normal(shape, dtype=np.float32)          # (this design's norms multiply by one plus the stored weight)
+            elif len(shape) == 1 and leaf in ("norm1", "norm2", "norm", "ls1", "ls2"):
                 a = 1.0 + 0.05 * rng.standard_normal(shape, dtype=np.float32)
             elif leaf == "dwa":
                 a = np.full(shape, 1.0 / shape[0], np.float32)
