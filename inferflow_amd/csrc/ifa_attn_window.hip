@@ -202,9 +202,11 @@ __global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_s
     float *Vs = Ks + WT_K * DKP;             // [32][DVP]
     float *Ps = Vs + WT_K * DVP;             // [4][32][33]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, i = lane & 31, g = lane >> 5;
-    const int h = blockIdx.y, kvh = h / (P.heads / P.kv_heads), dk = P.dim, dv = P.vdim;
-    // which sequence and which of its 128-row tiles
-    int tile = blockIdx.x, sq = 0;
+    const int h = blockIdx.x, kvh = h / (P.heads / P.kv_heads), dk = P.dim, dv = P.vdim;
+    // which sequence and which of its 128-row tiles.  The grid runs over (head, tile) with the head as the fast index and the tiles from
+    // the last one down: the tiles with the most key blocks start first, and the query heads of a group, which read the same key and
+    // value rows, run side by side.
+    int tile = (int)(gridDim.y - 1 - blockIdx.y), sq = 0;
     for (; sq < n_seqs; sq++) {
         const int nt = (P.seqs[sq].n + WT_Q - 1) / WT_Q;
         if (tile < nt) break;
@@ -436,7 +438,8 @@ static int attention_launch(const char *who, const void *q_f32, size_t ldq, int 
         const int NTK = (dim + 31) / 32, NTV = (vdim + 31) / 32;
         const size_t smem_t = ((size_t)(WT_Q + WT_K) * (32 * NTK + 1) + (size_t)WT_K * (32 * NTV + 1) + 4 * 32 * 33) * 4;
         const int vec = (dim % 4 == 0 && vdim % 4 == 0 && k_off % 4 == 0 && v_off % 4 == 0) ? 1 : 0;      // (arena bases are 256-byte aligned)
-        const dim3 grid((unsigned)tiles, (unsigned)heads);
+        IFA_REQUIRE(tiles < 65536, "%s: %zu query tiles in one step", who, tiles);
+        const dim3 grid((unsigned)heads, (unsigned)tiles);
 #define IFA_WT(K, V) { IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_attn_window_tile<K, V>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_t)); \
                        hipLaunchKernelGGL((k_attn_window_tile<K, V>), grid, dim3(256), smem_t, ifa_s(stream), P, n_seqs, vec); }
 #define IFA_WTV(K) { if (NTV == 1) IFA_WT(K, 1) else if (NTV == 2) IFA_WT(K, 2) else if (NTV == 3) IFA_WT(K, 3) else IFA_WT(K, 4) }
