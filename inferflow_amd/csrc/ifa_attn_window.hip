@@ -166,14 +166,16 @@ __global__ void __launch_bounds__(64) k_attn_window_combine(WinAttnArgs P)
     const float M = fmaxf(snk, wave_max(m_sp));
     const float f_sp = m_sp == -INFINITY ? 0.0f : expf(m_sp - M);
     const float L = wave_sum(l_sp * f_sp) + (has_sink(P) ? expf(snk - M) : 0.0f);
-    for (int d = lane; d < dim; d += 64) {
+    // (every lane walks every group of 64 columns, also where it has no column of its own: the scale factors come from other lanes)
+    for (int d0 = 0; d0 < dim; d0 += 64) {
+        const int d = d0 + lane;
         float v[WA_MAX_SPLITS];
 #pragma unroll
-        for (int sp = 0; sp < WA_MAX_SPLITS; sp++) v[sp] = sp < nsplit ? src[(size_t)sp * (dim + 2) + 2 + d] : 0.0f;
+        for (int sp = 0; sp < WA_MAX_SPLITS; sp++) v[sp] = (sp < nsplit && d < dim) ? src[(size_t)sp * (dim + 2) + 2 + d] : 0.0f;
         float o = 0.0f;
 #pragma unroll
         for (int sp = 0; sp < WA_MAX_SPLITS; sp++) o = fmaf(v[sp], __shfl(f_sp, sp, 64), o);
-        P.out[(size_t)t * P.ldo + (size_t)h * dim + d] = o / L;
+        if (d < dim) P.out[(size_t)t * P.ldo + (size_t)h * dim + d] = o / L;
     }
 }
 

@@ -164,6 +164,33 @@ def test_rotated_attention_in_portions_and_single_rows(heads, kv_heads, dim, vdi
     assert np.abs(res[0] - res[1]).max() > 1e-4 and np.abs(res[2] - res[1]).max() > 1e-4
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,rot_dims", [(2, 2, 40, 72, 40), (4, 1, 100, 100, 50), (2, 1, 16, 200, 8)])
+def test_single_rows_over_a_long_context_with_value_heads_that_end_inside_a_group_of_64_columns(heads, kv_heads, dim, vdim, rot_dims):
+    """1300 keys: the keys of a (row, head) are shared out to twenty workgroups, and the merge of their partial results walks value
+    columns 64 .. vdim - 1 with only some lanes holding a column"""
+    rng = np.random.default_rng(dim + vdim)
+    L, eps, scale, base, ctx = 1300, 1e-5, 0.3, 10000.0, 2001
+    q, k, v, qw, kw = attention_case(heads, kv_heads, dim, vdim, rot_dims, L, rng)
+    want = oracle_attention(q, k, v, qw, kw, heads, kv_heads, dim, vdim, rot_dims, base, scale, eps)
+    fr = freq_table(rot_dims, base)
+    k_off, v_off = 0, ctx * kv_heads * dim
+    sl = Slots(1, v_off + ctx * kv_heads * vdim)
+    ws = torch.full((heads * 32 * (vdim + 2),), float('nan'), dtype=torch.float32, device='cuda')
+    Lc = capi()
+    at = 0
+    for n in [1290] + [1] * 10:
+        d, rs, T = seq_tables([(n, at, 0)])
+        qd, kd, vd = dev32(q[at:at + n]), dev32(k[at:at + n]), dev32(v[at:at + n])
+        ia.check(Lc.ifa_qk_rope_store_f32(p(qd), heads * dim, heads, p(kd), kv_heads * dim, p(vd), kv_heads * vdim, kv_heads, dim, vdim, p(devbf(qw)), p(devbf(kw)), eps,
+                                          rot_dims, p(fr), p(d), p(rs), T, p(sl.table), k_off, v_off, None))
+        out = torch.empty((T, heads * vdim), dtype=torch.float32, device="cuda")
+        ia.check(Lc.ifa_attention_kv_f32(p(qd), heads * dim, heads, kv_heads, dim, vdim, scale, 0, 0, 1, 0.0, p(d), p(rs), T, p(sl.table), k_off, v_off, p(out),
+                                         heads * vdim, host_seqs([(n, at, 0)]), 1, 16, ctx, p(ws), ws.numel() * 4, None))
+        sync()
+        assert np.abs(out.cpu().numpy() - want[at:at + n]).max() < 2e-5 * max(1.0, np.abs(want).max()), (at, n)
+        at += n
+
+
 def test_rotated_attention_tiles_over_several_sequences():
     """one step holds a 150-token prompt, a single continued token and a 40-token continued portion: tiles must not cross sequences"""
     rng = np.random.default_rng(78)
