@@ -542,7 +542,7 @@ int ifa_attention_kv_f32(const void *q_f32, size_t ldq, int heads, int kv_heads,
 /* rows of a step: per head RMS norm over dim with a weight (bf16 [dim], shared by the heads; null: no norm), then rotation of the first
  * rot_dims dimensions, dimension i paired with i + rot_dims / 2: (u, v) -> (u cos a - v sin a, v cos a + u sin a), a = pos * freq[i]
  * (freq_f64_dev: double [rot_dims / 2], angles formed in double).  Query heads are rewritten in place; key heads go to the K rows of
- * the sequences' caches, the values as they are to the V rows.  k_f32 null: queries only.  dim <= 256. */
+ * the sequences' caches, the values as they are to the V rows.  k_f32 null: queries only.  dim <= 1024. */
 int ifa_qk_rope_store_f32(void *q_f32, size_t ldq, int heads, const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int kv_heads, int dim, int vdim,
                           const void *q_norm_w_bf16, const void *k_norm_w_bf16, float eps, int rot_dims, const double *freq_f64_dev, const void *seqs_dev,
                           const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off, ifa_stream stream);

@@ -342,6 +342,7 @@ __global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_s
 // (formed in double: at position 1000 one fp32 ulp of the angle is already 1e-4); the rest pass unchanged.  Query heads are rewritten in
 // place; key heads go into the K rows of the cache, the value heads (as projected) into its V rows.  k null: the row brings no keys
 // and values of its own (the layer reads another layer's cache rows).
+template <int RS_CPL>
 __global__ void __launch_bounds__(256) k_qk_rope_store(float *__restrict__ q, size_t ldq, int heads, const float *__restrict__ k, size_t ldk,
                                                        const float *__restrict__ v, size_t ldv, int kv_heads, int dim, int vdim,
                                                        const bf16_t *__restrict__ q_norm_w, const bf16_t *__restrict__ k_norm_w, float eps, int rot_dims,
@@ -370,10 +371,10 @@ __global__ void __launch_bounds__(256) k_qk_rope_store(float *__restrict__ q, si
             for (int c = lane; c < dim; c += 64) s = fmaf(src[c], src[c], s);
             r = 1.0f / sqrtf(wave_sum(s) / (float)dim + eps);
         }
-        // every lane reads both members of its pairs before anything of the head is written (q is rewritten in place); dim <= 256
-        float val[4], oth[4];
+        // every lane reads both members of its pairs before anything of the head is written (q is rewritten in place); dim <= 64 RS_CPL
+        float val[RS_CPL], oth[RS_CPL];
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
+        for (int e = 0; e < RS_CPL; e++) {
             const int c = lane + 64 * e;
             val[e] = oth[e] = 0.0f;
             if (c < dim) {
@@ -382,7 +383,7 @@ __global__ void __launch_bounds__(256) k_qk_rope_store(float *__restrict__ q, si
             }
         }
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
+        for (int e = 0; e < RS_CPL; e++) {
             const int c = lane + 64 * e;
             if (c >= dim) continue;
             float out = val[e];
@@ -500,12 +501,14 @@ int ifa_qk_rope_store_f32(void *q_f32, size_t ldq, int heads, const void *k_f32,
                           const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off, ifa_stream stream)
 {
     IFA_REQUIRE(q_f32 && seqs_dev && row_seq_dev && slot_base_dev && (!k_f32 || v_f32), "ifa_qk_rope_store_f32: null pointer");
-    IFA_REQUIRE(heads > 0 && kv_heads > 0 && dim > 0 && dim <= 256 && vdim > 0 && rows > 0 && rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0
+    IFA_REQUIRE(heads > 0 && kv_heads > 0 && dim > 0 && dim <= 1024 && vdim > 0 && rows > 0 && rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0
                 && (rot_dims == 0 || freq_f64_dev), "ifa_qk_rope_store_f32: bad shape (head size %d, %d rotated)", dim, rot_dims);
     IFA_REQUIRE(ldq >= (size_t)heads * dim && (!k_f32 || (ldk >= (size_t)kv_heads * dim && ldv >= (size_t)kv_heads * vdim)), "ifa_qk_rope_store_f32: row strides too small");
-    hipLaunchKernelGGL(k_qk_rope_store, dim3((unsigned)rows), dim3(256), (size_t)std::max(rot_dims, 2) * 4, ifa_s(stream), (float *)q_f32, ldq, heads, (const float *)k_f32, ldk,
-                       (const float *)v_f32, ldv, kv_heads, dim, vdim, (const bf16_t *)q_norm_w_bf16, (const bf16_t *)k_norm_w_bf16, eps, rot_dims, freq_f64_dev,
-                       (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, k_off, v_off);
+#define IFA_RS(N) hipLaunchKernelGGL(k_qk_rope_store<N>, dim3((unsigned)rows), dim3(256), (size_t)std::max(rot_dims, 2) * 4, ifa_s(stream), (float *)q_f32, ldq, heads, \
+                                     (const float *)k_f32, ldk, (const float *)v_f32, ldv, kv_heads, dim, vdim, (const bf16_t *)q_norm_w_bf16, (const bf16_t *)k_norm_w_bf16, eps, \
+                                     rot_dims, freq_f64_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, k_off, v_off)
+    if (dim <= 128) IFA_RS(2); else if (dim <= 256) IFA_RS(4); else IFA_RS(16);
+#undef IFA_RS
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -1060,7 +1060,7 @@ int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec
             IFA_REQUIRE(s.m_yarn_factor == 0.0f || (s.m_yarn_factor > 0.0f && s.m_yarn_original > 0.0f && s.m_yarn_fast > 0.0f && s.m_yarn_slow > 0.0f),
                         "ifa_model_create_layered: layer %d: bad frequency scaling", l);
         } else if (s.mixer == IFA_MIX_ROTARY) {
-            IFA_REQUIRE(s.a_heads > 0 && s.a_kv_heads > 0 && s.a_heads % s.a_kv_heads == 0 && s.a_dim > 0 && s.a_dim <= 256 && s.a_vdim > 0 && s.a_vdim <= 1024
+            IFA_REQUIRE(s.a_heads > 0 && s.a_kv_heads > 0 && s.a_heads % s.a_kv_heads == 0 && s.a_dim > 0 && s.a_dim <= 1024 && s.a_vdim > 0 && s.a_vdim <= 1024
                         && s.a_window >= 0 && s.a_keep_first >= 0 && s.a_rot_dims >= 0 && s.a_rot_dims <= s.a_dim && s.a_rot_dims % 2 == 0
                         && (s.a_rot_dims == 0 || s.a_rot_base > 1.0f), "ifa_model_create_layered: layer %d: bad attention sizes", l);
             if (s.a_kv_layer != 0) {

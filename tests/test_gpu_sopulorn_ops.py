@@ -122,7 +122,7 @@ def freq_table(rot_dims, base):
 
 @pytest.mark.parametrize("tile_min", [16, 1 << 30])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,rot_dims", [(4, 2, 24, 16, 24), (2, 2, 8, 40, 4), (3, 1, 68, 36, 30), (6, 3, 32, 32, 0), (2, 1, 128, 128, 128),
-                                                              (4, 1, 40, 72, 40), (1, 1, 5, 3, 2), (8, 2, 96, 8, 64), (2, 1, 160, 20, 100)])
+                                                              (4, 1, 40, 72, 40), (1, 1, 5, 3, 2), (8, 2, 96, 8, 64), (2, 1, 160, 20, 100), (2, 1, 320, 24, 200)])
 def test_rotated_attention_in_portions_and_single_rows(heads, kv_heads, dim, vdim, rot_dims, tile_min):
     rng = np.random.default_rng(heads + dim + vdim)
     L, eps, scale, base, ctx = 150, 1e-5, 0.3, 300.0, 160
