@@ -247,26 +247,47 @@ __global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_s
 #pragma unroll
     for (int r = 0; r < 16; r++) { m[r] = -INFINITY; l[r] = 0.0f; }
     float *Pw = Ps + wave * 32 * 33;
-    for (int b = 0; b < nb_keep + nb_win; b++) {
+    // 16-byte path: a thread stages NTK pieces of the key block and NTV of the value block; the pieces of block b + 1 are asked for
+    // before block b is worked on and wait in registers meanwhile, so that the loads run behind the matrix-core work
+    float4 kreg[NTK], vreg[NTV];
+    auto fetch = [&](int b) {
+        const bool kept = b < nb_keep;
+        const int kb0 = kept ? b * WT_K : lo_min + (b - nb_keep) * WT_K;
+        const int kc_n = kept ? min(WT_K, nkeep - kb0) : min(WT_K, p_last - kb0 + 1);
+#pragma unroll
+        for (int u = 0; u < NTK; u++) {
+            const int e = tid + 256 * u, row = e / (DK / 4), c4 = (e % (DK / 4)) * 4;
+            kreg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (row < kc_n && c4 < dk) kreg[u] = *reinterpret_cast<const float4 *>(kc + (size_t)(kb0 + row) * kvd + c4);
+        }
+#pragma unroll
+        for (int u = 0; u < NTV; u++) {
+            const int e = tid + 256 * u, row = e / (DV / 4), c4 = (e % (DV / 4)) * 4;
+            vreg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (row < kc_n && c4 < dv) vreg[u] = *reinterpret_cast<const float4 *>(vc + (size_t)(kb0 + row) * vvd + c4);
+        }
+    };
+    const int nb_all = nb_keep + nb_win;
+    if (vec && nb_all > 0) fetch(0);
+    for (int b = 0; b < nb_all; b++) {
         const bool kept = b < nb_keep;
         const int kb0 = kept ? b * WT_K : lo_min + (b - nb_keep) * WT_K;
         const int kc_n = kept ? min(WT_K, nkeep - kb0) : min(WT_K, p_last - kb0 + 1);
         __syncthreads();                 // the previous block's K / V reads are done (and Q is staged)
         if (vec) {
-            for (int e = tid; e < WT_K * (DK / 4); e += 256) {
-                const int row = e / (DK / 4), c4 = (e % (DK / 4)) * 4;
-                float4 kv = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (row < kc_n && c4 < dk) kv = *reinterpret_cast<const float4 *>(kc + (size_t)(kb0 + row) * kvd + c4);
+#pragma unroll
+            for (int u = 0; u < NTK; u++) {
+                const int e = tid + 256 * u, row = e / (DK / 4), c4 = (e % (DK / 4)) * 4;
                 float *kd = Ks + row * DKP + c4;
-                kd[0] = kv.x; kd[1] = kv.y; kd[2] = kv.z; kd[3] = kv.w;
+                kd[0] = kreg[u].x; kd[1] = kreg[u].y; kd[2] = kreg[u].z; kd[3] = kreg[u].w;
             }
-            for (int e = tid; e < WT_K * (DV / 4); e += 256) {
-                const int row = e / (DV / 4), c4 = (e % (DV / 4)) * 4;
-                float4 vv = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (row < kc_n && c4 < dv) vv = *reinterpret_cast<const float4 *>(vc + (size_t)(kb0 + row) * vvd + c4);
+#pragma unroll
+            for (int u = 0; u < NTV; u++) {
+                const int e = tid + 256 * u, row = e / (DV / 4), c4 = (e % (DV / 4)) * 4;
                 float *vd = Vs + row * DVP + c4;
-                vd[0] = vv.x; vd[1] = vv.y; vd[2] = vv.z; vd[3] = vv.w;
+                vd[0] = vreg[u].x; vd[1] = vreg[u].y; vd[2] = vreg[u].z; vd[3] = vreg[u].w;
             }
+            if (b + 1 < nb_all) fetch(b + 1);
         } else {
             for (int e = tid; e < WT_K * DK; e += 256) {
                 const int row = e / DK, c = e % DK;
