@@ -180,9 +180,10 @@ __global__ void __launch_bounds__(64) k_attn_window_combine(WinAttnArgs P)
 }
 
 // ---- prompts: 128 queries of one sequence per workgroup, the visible keys walked in blocks of 32 that are staged ONCE per workgroup
-// in LDS; each wave owns 32 queries: S = Q K^T and O += P V on the fp32 matrix cores (v_mfma_f32_32x32x2_f32: scores and weights
-// stay 32-bit), online softmax per query row (running maximum across the block's keys by lane exchange, the row sums kept per lane
-// and added up once at the end), P turned from the accumulator layout into an A operand through LDS.  dim = 32 NT.
+// in LDS; each wave owns 32 queries, one per lane of each half: S^T = K Q^T and O^T += V^T P^T on the fp32 matrix cores
+// (v_mfma_f32_32x32x2_f32: scores and weights stay 32-bit).  In the transposed products a lane's accumulators hold 16 keys of ITS
+// query, so the online softmax (running maximum, weights, rescaling of O^T) is lane-local but for one exchange between the halves,
+// and the weights are the second product's B operand as they lie in the accumulators: no trip through LDS.
 typedef float f32x16w __attribute__((ext_vector_type(16)));
 constexpr int WT_Q = 128, WT_K = 32;
 
@@ -202,7 +203,6 @@ __global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_s
     float *Qs = sm;                          // [128][DKP]
     float *Ks = Qs + WT_Q * DKP;             // [32][DKP]
     float *Vs = Ks + WT_K * DKP;             // [32][DVP]
-    float *Ps = Vs + WT_K * DVP;             // [4][32][33]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, i = lane & 31, g = lane >> 5;
     const int h = blockIdx.x, kvh = h / (P.heads / P.kv_heads), dk = P.dim, dv = P.vdim;
     // which sequence and which of its 128-row tiles.  The grid runs over (head, tile) with the head as the fast index and the tiles from
@@ -239,14 +239,11 @@ __global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_s
     const int lo_min = max(0, p0 - P.window + 1), nkeep = min(P.keep_first, lo_min), p_last = p0 + nq - 1;
     const int nb_keep = (nkeep + WT_K - 1) / WT_K, nb_win = (p_last - lo_min + 1 + WT_K - 1) / WT_K;
     f32x16w o[NTV];
-    float m[16], l[16];
+    float m = -INFINITY, l = 0.0f;          // of the lane's query (lane & 31)
 #pragma unroll
     for (int nt = 0; nt < NTV; nt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[nt][r] = 0.0f;
-#pragma unroll
-    for (int r = 0; r < 16; r++) { m[r] = -INFINITY; l[r] = 0.0f; }
-    float *Pw = Ps + wave * 32 * 33;
     // 16-byte path: a thread stages NTK pieces of the key block and NTV of the value block; the pieces of block b + 1 are asked for
     // before block b is worked on and wait in registers meanwhile, so that the loads run behind the matrix-core work
     float4 kreg[NTK], vreg[NTV];
@@ -301,60 +298,64 @@ __global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_s
         __syncthreads();
         const bool active = nq_w > 0 && kb0 <= qhi && (kept || kb0 + kc_n - 1 >= qlo - P.window + 1 || kb0 < P.keep_first);
         if (active) {
+            // S^T = K Q^T: the lane's 16 accumulators are 16 KEYS of ITS query (lane & 31), so the running maximum, the weights and the
+            // rescaling stay inside the lane but for one exchange between the two halves of the wave
             f32x16w acc;
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[r] = 0.0f;
             const float *qa = Qs + (32 * wave + i) * DKP + g, *ka = Ks + i * DKP + g;
 #pragma unroll 8
-            for (int s2 = 0; s2 < DK / 2; s2++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[2 * s2], ka[2 * s2], acc, 0, 0, 0);
-            const int j = kb0 + i;
-            const bool jin = i < kc_n;
+            for (int s2 = 0; s2 < DK / 2; s2++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[2 * s2], qa[2 * s2], acc, 0, 0, 0);
+            const int iq = qlo + i;
+            const bool qin = i < nq_w;
+            float mloc = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int q = (r & 3) + 8 * (r >> 2) + 4 * g, iq = qlo + q;
-                const bool vis = jin && q < nq_w && j <= iq && (iq - j < P.window || j < P.keep_first);
+                const int kk = (r & 3) + 8 * (r >> 2) + 4 * g, j = kb0 + kk;
+                const bool vis = qin && kk < kc_n && j <= iq && (iq - j < P.window || j < P.keep_first);
                 float sc = acc[r] * P.scale;
                 if (P.softcap > 0.0f) sc = P.softcap * tanhf(sc / P.softcap);
                 if (P.rel && vis) sc += bf2f(P.rel[(size_t)P.bucket_of[iq - j] * P.heads + h]);
                 sc = vis ? sc : -INFINITY;
-                const float m_new = fmaxf(m[r], half_wave_max(sc));
-                const float pr = vis ? expf(sc - m_new) : 0.0f;
-                const float corr = m[r] == -INFINITY ? 1.0f : expf(m[r] - m_new);      // (m_new == -inf only while nothing was visible: sums are 0)
-                l[r] = l[r] * corr + pr;
-                m[r] = m_new;
-#pragma unroll
-                for (int nt = 0; nt < NTV; nt++) o[nt][r] *= corr;
-                Pw[q * 33 + i] = pr;
+                acc[r] = sc;
+                mloc = fmaxf(mloc, sc);
             }
-        }
-        __syncthreads();                 // P of every wave is in LDS
-        if (active) {
-            const float *pa = Pw + i * 33 + g;
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            const float m_new = fmaxf(m, mloc);
+            const float corr = m == -INFINITY ? 1.0f : expf(m - m_new);      // (m_new == -inf only while nothing was visible: sums are 0)
+            float psum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) { acc[r] = acc[r] == -INFINITY ? 0.0f : expf(acc[r] - m_new); psum += acc[r]; }
+            l = l * corr + psum;             // (the keys of this half of the wave; the halves are added at the end)
+            m = m_new;
+            // O^T += V^T P^T: the weights are the B operand as they lie in the accumulators (step s2 takes keys (s2 & 3) + 8 (s2 >> 2) + 4 g)
 #pragma unroll
             for (int nt = 0; nt < NTV; nt++) {
-                const float *va = Vs + g * DVP + 32 * nt + i;
-#pragma unroll 8
-                for (int s2 = 0; s2 < WT_K / 2; s2++) o[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[2 * s2], va[2 * s2 * DVP], o[nt], 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[nt][r] *= corr;
+                const float *va = Vs + 4 * g * DVP + 32 * nt + i;
+#pragma unroll
+                for (int s2 = 0; s2 < 16; s2++)
+                    o[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[((s2 & 3) + 8 * (s2 >> 2)) * DVP], acc[s2], o[nt], 0, 0, 0);
             }
         }
     }
+    // the lane holds value columns 32 nt + (r & 3) + 8 (r >> 2) + 4 g of its query
     const float snk = sink_of(P, h);
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int q = (r & 3) + 8 * (r >> 2) + 4 * g;
-        float ls = l[r];
-#pragma unroll
-        for (int of = 16; of > 0; of >>= 1) ls += __shfl_xor(ls, of, 64);
-        if (q >= nq_w) continue;
-        const float M = fmaxf(m[r], snk);
-        const float f = expf(m[r] - M);
+    const float ls = l + __shfl_xor(l, 32, 64);
+    if (i < nq_w) {
+        const float M = fmaxf(m, snk);
+        const float f = expf(m - M);
         const float L = ls * f + (has_sink(P) ? expf(snk - M) : 0.0f);
         const float sc = f / L;
+        float *dst = P.out + (size_t)(r0 + 32 * wave + i) * P.ldo + (size_t)h * dv;
 #pragma unroll
-        for (int nt = 0; nt < NTV; nt++) {
-            const int c = 32 * nt + i;
-            if (c < dv) P.out[(size_t)(r0 + 32 * wave + q) * P.ldo + (size_t)h * dv + c] = o[nt][r] * sc;
-        }
+        for (int nt = 0; nt < NTV; nt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int c = 32 * nt + (r & 3) + 8 * (r >> 2) + 4 * g;
+                if (c < dv) dst[c] = o[nt][r] * sc;
+            }
     }
 }
 
@@ -460,7 +461,7 @@ static int attention_launch(const char *who, const void *q_f32, size_t ldq, int 
         size_t tiles = 0;
         for (int q = 0; q < n_seqs; q++) tiles += ((size_t)sh[q].n + WT_Q - 1) / WT_Q;
         const int NTK = (dim + 31) / 32, NTV = (vdim + 31) / 32;
-        const size_t smem_t = ((size_t)(WT_Q + WT_K) * (32 * NTK + 1) + (size_t)WT_K * (32 * NTV + 1) + 4 * 32 * 33) * 4;
+        const size_t smem_t = ((size_t)(WT_Q + WT_K) * (32 * NTK + 1) + (size_t)WT_K * (32 * NTV + 1)) * 4;
         const int vec = (dim % 4 == 0 && vdim % 4 == 0 && k_off % 4 == 0 && v_off % 4 == 0) ? 1 : 0;      // (arena bases are 256-byte aligned)
         IFA_REQUIRE(tiles < 65536, "%s: %zu query tiles in one step", who, tiles);
         const dim3 grid((unsigned)heads, (unsigned)tiles);
