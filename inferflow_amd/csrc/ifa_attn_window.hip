@@ -187,13 +187,6 @@ __global__ void __launch_bounds__(64) k_attn_window_combine(WinAttnArgs P)
 typedef float f32x16w __attribute__((ext_vector_type(16)));
 constexpr int WT_Q = 128, WT_K = 32;
 
-__device__ __forceinline__ float half_wave_max(float v)      // over the 32 lanes that share lane >> 5
-{
-#pragma unroll
-    for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-
 // Key rows of dim <= 32 NTK and value rows of vdim <= 32 NTV floats; the columns beyond are zero in LDS.
 template <int NTK, int NTV>
 __global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_seqs, int vec)
