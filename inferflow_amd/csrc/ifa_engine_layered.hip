@@ -87,6 +87,7 @@ struct LayeredNet {
     // wave repeats the element-wise work for its rows) and within 1 % at width 1024: off by default
     int opt_fuse_rows = 0;
     int opt_fuse_post = 1;                 // POSTNORM layers, steps of at most 8 rows: norm-add, depth average, next input convolution and its tail in one launch
+                                           // SANDWICH layers, every step size: the norm behind a sub-layer and the norm in front of the next one in one launch
     float *attn_ws = nullptr; size_t attn_ws_bytes = 0;      // partial results of the windowed attention when a (row, head)'s keys are shared out
     int opt_attn_tile_min = 16;            // steps of at least this many rows run the windowed attention through the tiled kernel
     std::vector<ifa_seq_desc> seqs_host;   // the current step's sequences (the tiled attention's grid is sized from them)
