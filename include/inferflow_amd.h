@@ -251,7 +251,9 @@ typedef struct {
 enum {
     IFA_T_EMBD = 0, IFA_T_OUT_NORM = 1, IFA_T_OUT_NORM_B = 2, IFA_T_LM_HEAD = 3,
     IFA_T_EMBD_NORM = 4,      /* layer-list models with stem 1: weight of the grouped RMS norm behind the embedding */
-    IFA_T_BIGRAM = 5,         /* layer-list models with stem 2: hashed token-pair embedding [bigram_buckets + 1][width] */
+    IFA_T_BIGRAM = 5,         /* layer-list models with stem 2 / 3: hashed token-pair embedding [bigram_buckets + 1][width] */
+    IFA_T_OUT_NORM_ALPHA = 6, /* layer-list models with stem 3: the scalar of the Dynamic Tanh norm before lm_head (its bias: IFA_T_OUT_NORM_B) */
+    IFA_T_LOOP_STEP = 7,      /* layer-list models with a looped layer group: [loop_times][width], row t added before pass t */
     IFA_T_ATTN_NORM = 10, IFA_T_ATTN_NORM_B = 11, IFA_T_WQ = 12, IFA_T_WK = 13, IFA_T_WV = 14, IFA_T_WO = 15,
     IFA_T_FFN_NORM = 16, IFA_T_FFN_NORM_B = 17, IFA_T_W1 = 18, IFA_T_W2 = 19, IFA_T_W3 = 20, IFA_T_MOE_GATE = 21,
     IFA_T_WQ_B = 22, IFA_T_WK_B = 23, IFA_T_WV_B = 24, IFA_T_WO_B = 25, IFA_T_W1_B = 26, IFA_T_W2_B = 27, IFA_T_W3_B = 28,
@@ -651,6 +653,61 @@ int ifa_moe_experts_gated_f32(const void *h_f32, size_t ldh, size_t rows, int wi
                               const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes, void *y_f32, size_t ldy,
                               int accumulate, ifa_stream stream);
 
+
+/* ---- ops of pre-norm blocks with element-wise norms, looped layer groups, rotated values and per-channel recurrences */
+/* Dynamic Tanh "norm": y[t][c] = tanh(alpha * x[t][c]) * w[c] + b[c]; alpha_bf16 one value, w / b bf16 [cols]; no mean, no variance */
+int ifa_dyt_f32(const void *x_f32, size_t ldx, size_t rows, size_t cols, const void *alpha_bf16, const void *w_bf16, const void *b_bf16, void *y_f32,
+                size_t ldy, ifa_stream stream);
+/* the residual update behind a sub-layer and the Dynamic Tanh in front of the next one in one launch: x += m (m null: skip), then
+ * (w not null) h = tanh(alpha x) w + b */
+int ifa_add_dyt_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *alpha_bf16, const void *w_bf16,
+                    const void *b_bf16, void *h_f32, size_t ldh, ifa_stream stream);
+/* x[t][c] += (add_f32 ? add[t][c] : 0) + (vec_bf16 ? vec[c] : 0): what a pass of a looped layer group starts from */
+int ifa_add_rows_vec_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *add_f32, size_t lda, const void *vec_bf16, ifa_stream stream);
+/* ifa_embed_pair_f32 with the token embedding multiplied by embed_scale (the pair row is not) and an optional second copy of the result */
+int ifa_embed_pair_scaled_f32(const void *embed_bf16, int vocab, int width, float embed_scale, const void *pair_bf16, int buckets, int mul_prev, int mul_cur,
+                              const int *tokens_dev, const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t state_off,
+                              void *x_f32, void *x_copy_f32, ifa_stream stream);
+/* ifa_qk_rope_store_f32 whose values are treated too before they enter the V rows: v_norm != 0: each value head is divided by its root
+ * mean square (eps, no weight); v_freq_f64_dev != null: the value head of position j then turns by j over ALL vdim dimensions, pair
+ * (m, m + vdim / 2) by j * v_freq[m] (double [vdim / 2]; vdim even). */
+int ifa_qkv_rope_store_f32(void *q_f32, size_t ldq, int heads, const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int kv_heads, int dim, int vdim,
+                           const void *q_norm_w_bf16, const void *k_norm_w_bf16, float eps, int rot_dims, const double *freq_f64_dev, int v_norm,
+                           const double *v_freq_f64_dev, const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off,
+                           size_t v_off, ifa_stream stream);
+/* heads of a step's rows turned in place by sign * position: pair (m, m + rot_dims / 2) of the first rot_dims dimensions of every head by
+ * sign * pos * freq[m] (angles in double).  sign -1 turns an attention output over rotated values back. */
+int ifa_rotate_heads_f32(void *x_f32, size_t ldx, int heads, int dim, int rot_dims, const double *freq_f64_dev, float sign, const void *seqs_dev,
+                         const int *row_seq_dev, size_t rows, ifa_stream stream);
+/* ifa_attention_kv_f32 with a learned sink per head (sink_bf16 [heads]; null: none): exp(sink_h) joins the denominator */
+int ifa_attention_kv_sinks_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int vdim, float scale, int window, int keep_first,
+                               const void *sink_bf16, const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off,
+                               size_t v_off, void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, int max_keys, void *ws_f32,
+                               size_t ws_bytes, ifa_stream stream);
+/* gates of the generalized delta rule, per row and key channel c of heads * dim: decay[c] = exp(-decay_mult * sigmoid(w2[c] . tanh(lr) + w0[c]))
+ * (lr fp32 [rows][rank]: the bottleneck's pre-activations; w2 bf16 [heads * dim][rank]; w0 bf16 [heads * dim], nullable), unit key
+ * u = k / sqrt(sum_head(k^2) + l2_eps), removal[c] = sigmoid(a[c]) * u[c] (a with its bias already added).  Outputs fp32 [rows][heads * dim], contiguous. */
+int ifa_chan_delta_gates_f32(const void *lr_f32, size_t ldl, int rank, const void *w2_bf16, const void *w0_bf16, float decay_mult, const void *a_f32, size_t lda,
+                             const void *k_f32, size_t ldk, int heads, int dim, float l2_eps, size_t rows, void *decay_f32, void *unit_f32, void *removal_f32,
+                             ifa_stream stream);
+/* generalized delta rule with a decay and a removal rate per key channel: per head, S [dk][dv] fp32 in the slot,
+ * S <- diag(decay_t) S - removal_t (unit_t^T S) + k_t v_t^T (both terms read the old state), o_t = S^T q_t.
+ * decay / unit / removal fp32 [rows][heads * dk] (row stride ldg).  dk <= 256. */
+int ifa_state_scan_chan_f32(const void *q_f32, size_t ldq, const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int heads, int dk, int dv,
+                            const void *decay_f32, const void *unit_f32, const void *removal_f32, size_t ldg, const void *seqs_dev, int n_seqs,
+                            void *const *slot_base_dev, size_t state_off, void *out_f32, size_t ldo, ifa_stream stream);
+/* Router with a choice of scores: score_kind 0 = softmax over all (ifa_moe_route_f32), 1 = sigmoid of each logit; the `top` largest
+ * (score + correction) are chosen (lowest index on ties), weights = their plain scores, not renormalized */
+int ifa_moe_route_scores_f32(int score_kind, const void *logits_f32, size_t ld, size_t rows, int n_all, int top, const void *correction_bf16, int *idx_dev,
+                             void *wgt_f32, ifa_stream stream);
+int ifa_moe_route_rows_scores_f32(int score_kind, const void *h_f32, size_t ldh, size_t rows, int width, const void *router_bf16, int n_all, int top,
+                                  const void *correction_bf16, int *idx_dev, void *wgt_f32, ifa_stream stream);
+/* Gated experts with a choice of the gate: glu_kind 0 = silu(gate) * up (ifa_moe_experts_gated_f32), 3 = the clamped form of ifa_glu_ex_f32
+ * (g = min(gate, limit), u = clamp(up, +-limit), g sigmoid(1.702 g) (u + 1)) */
+int ifa_moe_experts_glu_f32(int glu_kind, float limit, const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int top,
+                            const void *gate_up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
+                            void *y_f32, size_t ldy, int accumulate, ifa_stream stream);
+
 /* ======================================================================== */
 /* Layer-list worker: a decoder whose layers are given one by one, each with its own sequence mixer, a 32-bit residual       */
 /* stream and bfloat16 weights (csrc/ifa_engine_layered.hip).  It is an ifa_model: finalize / kv_slots / select_kv /        */
@@ -661,14 +718,18 @@ int ifa_moe_experts_gated_f32(const void *h_f32, size_t ldh, size_t rows, int wi
 enum { IFA_MIX_WINDOW_LINEAR = 1,   /* windowed softmax attention (values = keys as projected) + decayed linear attention, side by side */
        IFA_MIX_GATED_DELTA = 2,     /* gated delta rule behind short convolutions */
        IFA_MIX_LATENT = 3,          /* latent attention: one compressed key / value row per position, a rotated key part shared by all heads */
-       IFA_MIX_ROTARY = 4 };        /* softmax attention with rotated queries / keys: grouped queries, q | k | v projections with biases, weighted
+       IFA_MIX_ROTARY = 4,          /* softmax attention with rotated queries / keys: grouped queries, q | k | v projections with biases, weighted
                                      * RMS norm of q and k per head, rotation of the first a_rot_dims dimensions (pairs i, i + a_rot_dims / 2),
-                                     * values of their own size, optional sink of fixed score, optional window, keys / values of an earlier layer */
+                                     * values of their own size, optional sink (fixed score or learned per head), optional window, keys / values
+                                     * of an earlier layer, optionally scaled frequencies, normed values, rotated values */
+       IFA_MIX_CHAN_DELTA = 5 };    /* generalized delta rule: decay and removal rate per head and key channel (the decay through a small
+                                     * two-matrix bottleneck), unit keys for the removal, per-head RMS norm x weight x sigmoid gate on the output */
 /* wiring of a layer.  PARALLEL: h = norm1(x); x <- x + ls1 * mixer(h) + ls2 * ffn(h).  POSTNORM: the sub-layers read x itself (plus a
  * short causal convolution of x when canon_taps > 0) and the grouped RMS norm sits on their OUTPUT: x <- x + norm1(mixer(x'));
  * x <- x + norm2(ffn(x')); with depth_avg the next layer reads sum_j dwa[j] X_j over the embedding output X_0 and every layer result.
- * SANDWICH: an RMS norm with weight (1 + w) before AND after each sub-layer: x <- x + norm1b(mixer(norm1(x))); x <- x + norm2b(ffn(norm2(x))). */
-enum { IFA_BLOCK_PARALLEL = 0, IFA_BLOCK_POSTNORM = 1, IFA_BLOCK_SANDWICH = 2 };
+ * SANDWICH: an RMS norm with weight (1 + w) before AND after each sub-layer: x <- x + norm1b(mixer(norm1(x))); x <- x + norm2b(ffn(norm2(x))).
+ * PRENORM: x <- x + mixer(norm1(x)); x <- x + ffn(norm2(x)) with Dynamic Tanh norms tanh(alpha x) w + b (tensors IFA_LT_NORM1 / _B / _ALPHA). */
+enum { IFA_BLOCK_PARALLEL = 0, IFA_BLOCK_POSTNORM = 1, IFA_BLOCK_SANDWICH = 2, IFA_BLOCK_PRENORM = 3 };
 enum { IFA_FFN_GATED = 0,           /* gated feed-forward (GELU tanh, biases), width `ffn` */
        IFA_FFN_MOE = 1,             /* mixture of experts: x_experts experts of width x_ff + x_identity identity experts, x_top per token */
        IFA_FFN_CLAMPED = 2 };       /* width `ffn`, no biases: g = min(gate, f_limit), u = clamp(up, +-f_limit), y = down(g sigmoid(1.702 g) (u + 1)) */
@@ -703,6 +764,20 @@ typedef struct {
      * over the chosen logits; x_shared_ff > 0: a shared gated expert of that width for every row, times sigmoid(w_sg . h) */
     float f_limit;
     int x_gated, x_route, x_shared_ff;
+    /* more of IFA_MIX_ROTARY.  a_sink 2: a learned sink per head (tensor IFA_LT_A_SINK).  a_rot_scale_factor > 0: frequencies scaled by
+     * wavelength l = 2 pi / f: kept where l < original / high, f / factor where l > original / low, blended linearly in
+     * (original / l - low) / (high - low) between.  a_vnorm 1: value heads divided by their root mean square before they are cached.
+     * a_vrot 1: the value of position j enters the cache turned by j over all a_vdim dimensions (pairs m, m + a_vdim / 2, frequency
+     * a_rot_base^(-2m / a_vdim), never scaled) and the head's output at position i is turned back by -i. */
+    float a_rot_scale_factor, a_rot_scale_low, a_rot_scale_high, a_rot_scale_original;
+    int a_vnorm, a_vrot;
+    /* IFA_MIX_CHAN_DELTA: c_heads heads of c_dim key and value channels, bottleneck of c_rank for the decay; decay = exp(-c_decay_mult *
+     * sigmoid(.)); eps inside the root of the unit key */
+    int c_heads, c_dim, c_rank;
+    float c_decay_mult, c_l2_eps;
+    /* mixture: x_score 0 softmax over all, 1 sigmoid per expert (x_route 0); x_glu 0 silu(gate) * up, 3 the clamped form with x_limit (x_gated 1) */
+    int x_score, x_glu;
+    float x_limit;
 } ifa_layer_spec;
 typedef struct {
     int width, vocab, max_ctx, n_layers, device;
@@ -716,6 +791,13 @@ typedef struct {
      * bigram_buckets; row bigram_buckets for a sequence's first token; bigram_buckets 0: none), no position vector, RMS norm with
      * weight (1 + w) before lm_head.  The previous token of a sequence is kept in its slot. */
     int bigram_buckets, bigram_mul_prev, bigram_mul_cur;
+    /* stem 3: stem 2 with the token embedding times embed_scale (0: 1), a Dynamic Tanh norm before lm_head (IFA_T_OUT_NORM / _B / _ALPHA)
+     * and logits times logit_scale (0: 1) */
+    float embed_scale, logit_scale;
+    /* looped layer group: layers [loop_start, loop_stop) run loop_times times in a row with the same weights, each pass on cache rows and
+     * states of its own; before every pass but the first the embedding output is added to the residual, and before every pass row t of
+     * IFA_T_LOOP_STEP ([loop_times][width]).  loop_times 0: no group. */
+    int loop_start, loop_stop, loop_times;
 } ifa_layered_config;
 /* tensors of a layer-list model (global ones use IFA_T_EMBD / IFA_T_OUT_NORM / IFA_T_LM_HEAD with layer = -1) */
 enum {
@@ -730,6 +812,8 @@ enum {
     IFA_LT_NORM1B, IFA_LT_NORM2B,                  /* SANDWICH: the norms behind the sub-layers */
     IFA_LT_A_V, IFA_LT_A_Q_B, IFA_LT_A_K_B, IFA_LT_A_V_B, IFA_LT_A_Q_NORM, IFA_LT_A_K_NORM,      /* IFA_MIX_ROTARY (with IFA_LT_A_Q / _K / _O) */
     IFA_LT_X_ROUTER_B, IFA_LT_X_SH_GATE, IFA_LT_X_SH_UP, IFA_LT_X_SH_DOWN, IFA_LT_X_SH_SG,
+    IFA_LT_NORM1_B, IFA_LT_NORM1_ALPHA, IFA_LT_NORM2_B, IFA_LT_NORM2_ALPHA,                       /* PRENORM: bias and scalar of the Dynamic Tanh norms */
+    IFA_LT_C_R, IFA_LT_C_K, IFA_LT_C_V, IFA_LT_C_G, IFA_LT_C_A, IFA_LT_C_A_B, IFA_LT_C_W1, IFA_LT_C_W2, IFA_LT_C_W0, IFA_LT_C_NORM, IFA_LT_C_O,      /* IFA_MIX_CHAN_DELTA */
     IFA_LT_END
 };
 int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec *layers, ifa_model **out);

@@ -357,20 +357,31 @@ __global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_s
 // (formed in double: at position 1000 one fp32 ulp of the angle is already 1e-4); the rest pass unchanged.  Query heads are rewritten in
 // place; key heads go into the K rows of the cache, the value heads (as projected) into its V rows.  k null: the row brings no keys
 // and values of its own (the layer reads another layer's cache rows).
-template <int RS_CPL>
+// VX: the values are treated too (v_norm: each value head divided by its root mean square; v_freq: the head then turns by the row's position over
+// all vdim dimensions, pair (m, m + vdim / 2) by pos * v_freq[m]) instead of entering the V rows as projected.
+template <int RS_CPL, bool VX>
 __global__ void __launch_bounds__(256) k_qk_rope_store(float *__restrict__ q, size_t ldq, int heads, const float *__restrict__ k, size_t ldk,
                                                        const float *__restrict__ v, size_t ldv, int kv_heads, int dim, int vdim,
                                                        const bf16_t *__restrict__ q_norm_w, const bf16_t *__restrict__ k_norm_w, float eps, int rot_dims,
                                                        const double *__restrict__ freq, const SeqDesc *__restrict__ seqs, const int *__restrict__ row_seq,
-                                                       float *const *__restrict__ slot_base, size_t k_off, size_t v_off)
+                                                       float *const *__restrict__ slot_base, size_t k_off, size_t v_off, int v_norm,
+                                                       const double *__restrict__ v_freq)
 {
-    extern __shared__ float cs[];          // [rot_dims / 2] cos, [rot_dims / 2] sin
+    extern __shared__ float cs[];          // [rot_dims / 2] cos, [rot_dims / 2] sin; VX: [vdim / 2] cos, [vdim / 2] sin behind them
     const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
     const SeqDesc sd = seqs[row_seq[t]];
     const int pos = sd.pos0 + t - sd.row0, half = rot_dims / 2;
     for (int i = tid; i < half; i += blockDim.x) {
         const double a = (double)pos * freq[i];
         cs[i] = (float)cos(a); cs[half + i] = (float)sin(a);
+    }
+    float *vcs = cs + 2 * half;
+    const int vhalf = vdim / 2;
+    if (VX && k && v_freq) {
+        for (int i = tid; i < vhalf; i += blockDim.x) {
+            const double a = (double)pos * v_freq[i];
+            vcs[i] = (float)cos(a); vcs[vhalf + i] = (float)sin(a);
+        }
     }
     __syncthreads();
     const int n_items = heads + (k ? kv_heads : 0);
@@ -409,10 +420,57 @@ __global__ void __launch_bounds__(256) k_qk_rope_store(float *__restrict__ q, si
             dst[c] = out;
         }
     }
+    if (VX) {
+        if (!k) return;
+        // a wave per value head: weightless RMS norm, then the turn by the position (a lane reads both members of a pair from the input row)
+        for (int hd = wave; hd < kv_heads; hd += nw) {
+            const float *src = v + (size_t)t * ldv + (size_t)hd * vdim;
+            float *dst = slot_base[sd.slot] + v_off + ((size_t)pos * kv_heads + hd) * vdim;
+            float r = 1.0f;
+            if (v_norm) {
+                float s = 0.0f;
+                for (int c = lane; c < vdim; c += 64) s = fmaf(src[c], src[c], s);
+                r = 1.0f / sqrtf(wave_sum(s) / (float)vdim + eps);
+            }
+            for (int c = lane; c < vdim; c += 64) {
+                float out = src[c] * r;
+                if (v_freq && c < 2 * vhalf) {
+                    const int fi = c < vhalf ? c : c - vhalf;
+                    const float oth = src[c < vhalf ? c + vhalf : c - vhalf] * r;
+                    out = c < vhalf ? out * vcs[fi] - oth * vcs[vhalf + fi] : out * vcs[fi] + oth * vcs[vhalf + fi];
+                }
+                dst[c] = out;
+            }
+        }
+        return;
+    }
     if (k) {
         float *vd = slot_base[sd.slot] + v_off + (size_t)pos * kv_heads * vdim;
         const float *vs = v + (size_t)t * ldv;
         for (int c = tid; c < kv_heads * vdim; c += blockDim.x) vd[c] = vs[c];
+    }
+}
+
+// heads of a row turned in place by sign * position over their first rot_dims dimensions, pairs (m, m + rot_dims / 2); a workgroup per row
+__global__ void __launch_bounds__(256) k_rotate_heads(float *__restrict__ x, size_t ldx, int heads, int dim, int rot_dims, const double *__restrict__ freq, float sign,
+                                                      const SeqDesc *__restrict__ seqs, const int *__restrict__ row_seq)
+{
+    extern __shared__ float cs[];          // [rot_dims / 2] cos, [rot_dims / 2] sin
+    const int t = blockIdx.x, tid = threadIdx.x, half = rot_dims / 2;
+    const SeqDesc sd = seqs[row_seq[t]];
+    const int pos = sd.pos0 + t - sd.row0;
+    for (int i = tid; i < half; i += blockDim.x) {
+        const double a = (double)sign * (double)pos * freq[i];
+        cs[i] = (float)cos(a); cs[half + i] = (float)sin(a);
+    }
+    __syncthreads();
+    float *xr = x + (size_t)t * ldx;
+    for (int e = tid; e < heads * half; e += blockDim.x) {      // a thread owns a pair: both members read before either is written
+        const int hd = e / half, i = e % half;
+        float *p = xr + (size_t)hd * dim;
+        const float u = p[i], w = p[i + half];
+        p[i] = u * cs[i] - w * cs[half + i];
+        p[i + half] = w * cs[i] + u * cs[half + i];
     }
 }
 
@@ -519,13 +577,56 @@ int ifa_qk_rope_store_f32(void *q_f32, size_t ldq, int heads, const void *k_f32,
     IFA_REQUIRE(heads > 0 && kv_heads > 0 && dim > 0 && dim <= 1024 && vdim > 0 && rows > 0 && rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0
                 && (rot_dims == 0 || freq_f64_dev), "ifa_qk_rope_store_f32: bad shape (head size %d, %d rotated)", dim, rot_dims);
     IFA_REQUIRE(ldq >= (size_t)heads * dim && (!k_f32 || (ldk >= (size_t)kv_heads * dim && ldv >= (size_t)kv_heads * vdim)), "ifa_qk_rope_store_f32: row strides too small");
-#define IFA_RS(N) hipLaunchKernelGGL(k_qk_rope_store<N>, dim3((unsigned)rows), dim3(256), (size_t)std::max(rot_dims, 2) * 4, ifa_s(stream), (float *)q_f32, ldq, heads, \
+#define IFA_RS(N) hipLaunchKernelGGL((k_qk_rope_store<N, false>), dim3((unsigned)rows), dim3(256), (size_t)std::max(rot_dims, 2) * 4, ifa_s(stream), (float *)q_f32, ldq, heads, \
                                      (const float *)k_f32, ldk, (const float *)v_f32, ldv, kv_heads, dim, vdim, (const bf16_t *)q_norm_w_bf16, (const bf16_t *)k_norm_w_bf16, eps, \
-                                     rot_dims, freq_f64_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, k_off, v_off)
+                                     rot_dims, freq_f64_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, k_off, v_off, 0, (const double *)nullptr)
     if (dim <= 128) IFA_RS(2); else if (dim <= 256) IFA_RS(4); else IFA_RS(16);
 #undef IFA_RS
     IFA_LAUNCH_CHECK();
     return IFA_OK;
+}
+
+int ifa_qkv_rope_store_f32(void *q_f32, size_t ldq, int heads, const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int kv_heads, int dim, int vdim,
+                           const void *q_norm_w_bf16, const void *k_norm_w_bf16, float eps, int rot_dims, const double *freq_f64_dev, int v_norm,
+                           const double *v_freq_f64_dev, const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off,
+                           size_t v_off, ifa_stream stream)
+{
+    IFA_REQUIRE(q_f32 && seqs_dev && row_seq_dev && slot_base_dev && (!k_f32 || v_f32), "ifa_qkv_rope_store_f32: null pointer");
+    IFA_REQUIRE(heads > 0 && kv_heads > 0 && dim > 0 && dim <= 1024 && vdim > 0 && vdim <= 4096 && rows > 0 && rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0
+                && (rot_dims == 0 || freq_f64_dev) && (!v_freq_f64_dev || vdim % 2 == 0), "ifa_qkv_rope_store_f32: bad shape (head sizes %d / %d, %d rotated)", dim, vdim, rot_dims);
+    IFA_REQUIRE(ldq >= (size_t)heads * dim && (!k_f32 || (ldk >= (size_t)kv_heads * dim && ldv >= (size_t)kv_heads * vdim)), "ifa_qkv_rope_store_f32: row strides too small");
+    const size_t smem = ((size_t)std::max(rot_dims, 2) + (size_t)vdim + 2) * 4;
+#define IFA_RS(N) hipLaunchKernelGGL((k_qk_rope_store<N, true>), dim3((unsigned)rows), dim3(256), smem, ifa_s(stream), (float *)q_f32, ldq, heads, \
+                                     (const float *)k_f32, ldk, (const float *)v_f32, ldv, kv_heads, dim, vdim, (const bf16_t *)q_norm_w_bf16, (const bf16_t *)k_norm_w_bf16, eps, \
+                                     rot_dims, freq_f64_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, k_off, v_off, v_norm ? 1 : 0, v_freq_f64_dev)
+    if (dim <= 128) IFA_RS(2); else if (dim <= 256) IFA_RS(4); else IFA_RS(16);
+#undef IFA_RS
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_rotate_heads_f32(void *x_f32, size_t ldx, int heads, int dim, int rot_dims, const double *freq_f64_dev, float sign, const void *seqs_dev,
+                         const int *row_seq_dev, size_t rows, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && seqs_dev && row_seq_dev && (rot_dims == 0 || freq_f64_dev), "ifa_rotate_heads_f32: null pointer");
+    IFA_REQUIRE(heads > 0 && dim > 0 && rows > 0 && rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && rot_dims <= 8192 && ldx >= (size_t)heads * dim,
+                "ifa_rotate_heads_f32: bad shape (head size %d, %d rotated)", dim, rot_dims);
+    if (rot_dims == 0) return IFA_OK;
+    hipLaunchKernelGGL(k_rotate_heads, dim3((unsigned)rows), dim3(256), (size_t)rot_dims * 4, ifa_s(stream), (float *)x_f32, ldx, heads, dim, rot_dims, freq_f64_dev, sign,
+                       (const SeqDesc *)seqs_dev, row_seq_dev);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_attention_kv_sinks_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int vdim, float scale, int window, int keep_first,
+                               const void *sink_bf16, const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off,
+                               size_t v_off, void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, int max_keys, void *ws_f32,
+                               size_t ws_bytes, ifa_stream stream)
+{
+    const int win = window > 0 ? window : (1 << 30);
+    return attention_launch("ifa_attention_kv_sinks_f32", q_f32, ldq, heads, kv_heads, dim, vdim, 0, 0.0f, scale, 0.0f, win, keep_first, nullptr, nullptr, 0, sink_bf16,
+                            0, 0.0f, seqs_dev, row_seq_dev, rows, slot_base_dev, k_off, v_off, out_f32, ldo, seqs_host, n_seqs, tile_min_rows, max_keys, ws_f32, ws_bytes,
+                            stream);
 }
 
 } // extern "C"

@@ -24,6 +24,12 @@
 // V rows of their own size; a layer may read the rows an earlier layer has written instead of projecting keys and values), and feed
 // forward through the clamped gated form or a mixture of gated experts with a router on the logits and a shared, sigmoid-gated expert.
 // Stem 2 adds a hashed token-pair embedding whose previous token lives in the slot.
+// Layers wired IFA_BLOCK_PRENORM put a Dynamic Tanh norm (tanh(alpha x) w + b) in front of each sub-layer (x <- x + mixer(norm1(x)),
+// x <- x + ffn(norm2(x))), mix with the rotary attention (here with a learned sink per head, a sliding window, scaled frequencies, normed
+// values that enter the cache turned by their position and an output turned back) or with the generalized delta rule (IFA_MIX_CHAN_DELTA:
+// state S [dim][dim] per head in the slot), and feed forward through a mixture of clamped gated experts chosen by sigmoid scores.
+// A looped layer group runs several times with the same weights: every pass has cache rows and states of its own (a layer's part of the
+// arena is repeated per pass), so the stack is walked as a list of RUNS (layer, pass); stem 3 keeps the embedding output for the passes.
 #include <algorithm>
 #include <cmath>
 #include <cstring>
@@ -56,6 +62,10 @@ struct LLayer {
     // expert's gate logit | shared gate | shared up) with its bias vector and column offsets
     size_t c_av = 0;
     bf16_t *w_in2 = nullptr, *b_in2 = nullptr; size_t n_in2 = 0, c2_fg = 0, c2_router = 0, c2_sg = 0, c2_shg = 0;
+    // PRENORM: frequencies of the rotated values; generalized delta rule: columns of r | k | v | g | a | bottleneck in the fused product;
+    // a layer of a looped group repeats its part of the arena per pass, pass_stride floats apart
+    double *freq_v = nullptr;
+    size_t c_cr = 0, c_ck = 0, c_cv = 0, c_cg = 0, c_ca = 0, c_cw = 0, pass_stride = 0;
     LTensor &T(int id) { return t[id - IFA_LT_NORM1]; }
     const LTensor &T(int id) const { return t[id - IFA_LT_NORM1]; }
 };
@@ -67,7 +77,9 @@ constexpr int MAX_SLOTS = 4096;
 struct LayeredNet {
     ifa_layered_config cfg;
     std::vector<LLayer> layers;
-    LTensor embd, out_norm, lm_head, embd_norm, bigram;
+    LTensor embd, out_norm, lm_head, embd_norm, bigram, out_norm_b, out_norm_alpha, loop_step;
+    std::vector<std::pair<int, int>> runs;          // the stack as it is walked: (layer, pass of the looped group or 0)
+    float *x0 = nullptr, *cg_decay = nullptr, *cg_unit = nullptr, *cg_rem = nullptr; size_t chan_max = 0;      // embedding output (looped group); gates of the generalized delta rule
     size_t arena_floats = 0, o_prev = 0;          // (o_prev: the cell of the sequence's last token, stem 2)
     std::vector<float *> slot_ptr;       // host copy of the table (null: not allocated yet)
     float **slot_base_dev = nullptr;
@@ -119,14 +131,25 @@ bool expected_shape(const LayeredNet *n, const ifa_layer_spec &s, int li, int id
     const size_t W = (size_t)n->cfg.width;
     vec = false;
     const bool par = s.mixer == IFA_MIX_WINDOW_LINEAR, del = s.mixer == IFA_MIX_GATED_DELTA, lat = s.mixer == IFA_MIX_LATENT, rot = s.mixer == IFA_MIX_ROTARY;
-    const bool post = s.block == IFA_BLOCK_POSTNORM, sand = s.block == IFA_BLOCK_SANDWICH, moe = has_moe(s);
+    const bool post = s.block == IFA_BLOCK_POSTNORM, sand = s.block == IFA_BLOCK_SANDWICH, pre = s.block == IFA_BLOCK_PRENORM, moe = has_moe(s);
+    const bool chan = s.mixer == IFA_MIX_CHAN_DELTA;
+    const size_t CH = (size_t)s.c_heads * s.c_dim;
     const bool own_kv = rot && s.a_kv_layer == 0, gated = s.ffn > 0 && s.ffn_kind == IFA_FFN_GATED, any_ffn = s.ffn > 0 || moe;
     const size_t SF = (size_t)s.x_shared_ff;
     const size_t MH = (size_t)s.m_heads, MQ = MH * (size_t)(s.m_dim + s.m_rot_dim), MR = (size_t)s.m_kv_rank, XA = (size_t)(s.x_experts + s.x_identity);
     switch (id) {
     case IFA_LT_NORM1: r = 1; c = W; vec = true; return true;
-    case IFA_LT_LS1: r = 1; c = W; vec = true; return !post && !sand;
-    case IFA_LT_NORM2: r = 1; c = W; vec = true; return (post && moe) || (sand && any_ffn);
+    case IFA_LT_LS1: r = 1; c = W; vec = true; return !post && !sand && !pre;
+    case IFA_LT_NORM2: r = 1; c = W; vec = true; return (post && moe) || ((sand || pre) && any_ffn);
+    case IFA_LT_NORM1_B: r = 1; c = W; vec = true; return pre;
+    case IFA_LT_NORM1_ALPHA: r = 1; c = 1; vec = true; return pre;
+    case IFA_LT_NORM2_B: r = 1; c = W; vec = true; return pre && any_ffn;
+    case IFA_LT_NORM2_ALPHA: r = 1; c = 1; vec = true; return pre && any_ffn;
+    case IFA_LT_C_R: case IFA_LT_C_K: case IFA_LT_C_V: case IFA_LT_C_G: case IFA_LT_C_A: r = CH; c = W; return chan;
+    case IFA_LT_C_A_B: case IFA_LT_C_W0: case IFA_LT_C_NORM: r = 1; c = CH; vec = true; return chan;
+    case IFA_LT_C_W1: r = (size_t)s.c_rank; c = W; return chan;
+    case IFA_LT_C_W2: r = CH; c = (size_t)s.c_rank; return chan;
+    case IFA_LT_C_O: r = W; c = CH; return chan;
     case IFA_LT_NORM1B: r = 1; c = W; vec = true; return sand;
     case IFA_LT_NORM2B: r = 1; c = W; vec = true; return sand && any_ffn;
     case IFA_LT_A_V: r = (size_t)s.a_kv_heads * s.a_vdim; c = W; return own_kv;
@@ -163,7 +186,7 @@ bool expected_shape(const LayeredNet *n, const ifa_layer_spec &s, int li, int id
     case IFA_LT_A_Q: r = (size_t)s.a_heads * s.a_dim; c = W; return par || rot;
     case IFA_LT_A_K: r = (size_t)s.a_kv_heads * s.a_dim; c = W; return par || own_kv;
     case IFA_LT_A_REL: r = (size_t)s.a_buckets; c = (size_t)s.a_heads; return par;
-    case IFA_LT_A_SINK: r = 1; c = (size_t)s.a_heads; vec = true; return par;
+    case IFA_LT_A_SINK: r = 1; c = (size_t)s.a_heads; vec = true; return par || (rot && s.a_sink == 2);
     case IFA_LT_A_O: r = W; c = (size_t)s.a_heads * (rot ? s.a_vdim : s.a_dim); return par || rot;
     case IFA_LT_L_Q: case IFA_LT_L_K: r = (size_t)s.l_heads * s.l_dim; c = W; return par;
     case IFA_LT_L_V: case IFA_LT_L_G: r = (size_t)s.l_heads * s.l_vdim; c = W; return par;
@@ -251,6 +274,13 @@ int ensure_rows(ifa_model *m, size_t T, size_t nseq)
         }
         lay_free(n->m4); lay_free(n->m5); lay_free(n->stack); lay_free(n->moe_wgt); lay_free(n->moe_idx); lay_free(n->moe_ws);
         n->m4 = n->m5 = n->stack = n->moe_wgt = nullptr; n->moe_idx = nullptr; n->moe_ws = nullptr; n->moe_ws_bytes = 0;
+        lay_free(n->x0); lay_free(n->cg_decay); lay_free(n->cg_unit); lay_free(n->cg_rem);
+        n->x0 = n->cg_decay = n->cg_unit = n->cg_rem = nullptr;
+        if (n->cfg.loop_times > 1) IFA_HIP_CHECK(hipMalloc((void **)&n->x0, T * W * 4));
+        if (n->chan_max) {
+            float **gb[] = {&n->cg_decay, &n->cg_unit, &n->cg_rem};
+            for (float **b : gb) IFA_HIP_CHECK(hipMalloc((void **)b, T * n->chan_max * 4));
+        }
         if (n->any_latent) { IFA_HIP_CHECK(hipMalloc((void **)&n->m4, T * n->mix_max * 4)); IFA_HIP_CHECK(hipMalloc((void **)&n->m5, T * n->mix_max * 4)); }
         if (n->any_depth_avg) IFA_HIP_CHECK(hipMalloc((void **)&n->stack, (n->layers.size() + 1) * T * W * 4));
         if (n->any_moe) {
@@ -447,6 +477,60 @@ int run_sandwich_layer(ifa_model *m, LLayer &L, size_t T, int nseq, bool h_ready
     return close_sub(n->m2, L.T(IFA_LT_NORM2B).data, next_norm);
 }
 
+// one PRENORM layer over T rows: x <- x + mixer(dyt1(x)); x <- x + experts(dyt2(x)), dyt(x) = tanh(alpha x) w + b.  pass: which copy of the
+// layer's cache rows / state (a layer of a looped group has one per pass).  The output products and the experts add into the residual themselves.
+int run_prenorm_layer(ifa_model *m, LLayer &L, size_t T, int nseq, int pass)
+{
+    LayeredNet *n = m->lay;
+    const ifa_layered_config &c = n->cfg;
+    const ifa_layer_spec &sp = L.spec;
+    const size_t W = (size_t)c.width, NI = L.n_in, po = (size_t)pass * L.pass_stride;
+    ifa_stream s = (ifa_stream)m->stream;
+    void *const *slots = (void *const *)n->slot_base_dev;
+    int rc;
+    if ((rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM1_ALPHA).data, L.T(IFA_LT_NORM1).data, L.T(IFA_LT_NORM1_B).data, n->h, W, s))) return rc;
+    if ((rc = linear(m, L.w_in, NI, W, n->h, W, T, L.b_in, nullptr, 1.0f, 0, n->proj, NI))) return rc;
+    if (sp.mixer == IFA_MIX_ROTARY) {
+        const int H = sp.a_heads, G = sp.a_kv_heads, D = sp.a_dim, DV = sp.a_vdim;
+        const size_t OV = (size_t)H * DV;
+        if ((rc = ifa_qkv_rope_store_f32(n->proj + L.c_aq, NI, H, n->proj + L.c_ak, NI, n->proj + L.c_av, NI, G, D, DV, L.T(IFA_LT_A_Q_NORM).data, L.T(IFA_LT_A_K_NORM).data,
+                                         c.eps, sp.a_rot_dims, L.freq, sp.a_vnorm, sp.a_vrot ? L.freq_v : nullptr, n->seqs_dev, n->row_seq_dev, T, slots, L.o_k + po,
+                                         L.o_v + po, s))) return rc;
+        if (sp.a_sink == 2)
+            rc = ifa_attention_kv_sinks_f32(n->proj + L.c_aq, NI, H, G, D, DV, sp.a_scale, sp.a_window, sp.a_keep_first, L.T(IFA_LT_A_SINK).data, n->seqs_dev, n->row_seq_dev, T,
+                                            slots, L.o_k + po, L.o_v + po, n->m1, OV, n->seqs_host.data(), (int)n->seqs_host.size(), n->opt_attn_tile_min, c.max_ctx, n->attn_ws,
+                                            n->attn_ws_bytes, s);
+        else
+            rc = ifa_attention_kv_f32(n->proj + L.c_aq, NI, H, G, D, DV, sp.a_scale, sp.a_window, sp.a_keep_first, sp.a_sink, sp.a_sink_score, n->seqs_dev, n->row_seq_dev, T,
+                                      slots, L.o_k + po, L.o_v + po, n->m1, OV, n->seqs_host.data(), (int)n->seqs_host.size(), n->opt_attn_tile_min, c.max_ctx, n->attn_ws,
+                                      n->attn_ws_bytes, s);
+        if (rc) return rc;
+        // the sum over values that entered the cache turned by their positions is turned back by the row's own position
+        if (sp.a_vrot && (rc = ifa_rotate_heads_f32(n->m1, OV, H, DV, DV & ~1, L.freq_v, -1.0f, n->seqs_dev, n->row_seq_dev, T, s))) return rc;
+        if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_A_O).data, W, OV, n->m1, OV, T, nullptr, nullptr, 1.0f, 1, n->x, W))) return rc;
+    } else {
+        const int H = sp.c_heads, D = sp.c_dim;
+        const size_t CH = (size_t)H * D;
+        if ((rc = ifa_chan_delta_gates_f32(n->proj + L.c_cw, NI, sp.c_rank, L.T(IFA_LT_C_W2).data, L.T(IFA_LT_C_W0).data, sp.c_decay_mult, n->proj + L.c_ca, NI,
+                                           n->proj + L.c_ck, NI, H, D, sp.c_l2_eps, T, n->cg_decay, n->cg_unit, n->cg_rem, s))) return rc;
+        if ((rc = ifa_state_scan_chan_f32(n->proj + L.c_cr, NI, n->proj + L.c_ck, NI, n->proj + L.c_cv, NI, H, D, D, n->cg_decay, n->cg_unit, n->cg_rem, CH, n->seqs_dev, nseq,
+                                          slots, L.o_rec + po, n->m1, CH, s))) return rc;
+        if ((rc = ifa_gated_groupnorm_f32(n->m1, CH, T, (int)CH, D, L.T(IFA_LT_C_NORM).data, (int)CH, n->proj + L.c_cg, NI, 0, c.eps, n->m1, CH, s))) return rc;
+        if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_C_O).data, W, CH, n->m1, CH, T, nullptr, nullptr, 1.0f, 1, n->x, W))) return rc;
+    }
+    if (!has_moe(sp)) return IFA_OK;
+    if ((rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM2_ALPHA).data, L.T(IFA_LT_NORM2).data, L.T(IFA_LT_NORM2_B).data, n->h, W, s))) return rc;
+    const int XA = sp.x_experts;
+    if (T <= 8 && XA <= 512) {      // a few rows: the router's product inside the choice's launch
+        if ((rc = ifa_moe_route_rows_scores_f32(sp.x_score, n->h, W, T, (int)W, L.T(IFA_LT_X_ROUTER).data, XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
+    } else {
+        if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_X_ROUTER).data, (size_t)XA, W, n->h, W, T, nullptr, nullptr, 1.0f, 0, n->m2, (size_t)XA))) return rc;
+        if ((rc = ifa_moe_route_scores_f32(sp.x_score, n->m2, (size_t)XA, T, XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
+    }
+    return ifa_moe_experts_glu_f32(sp.x_glu, sp.x_limit, n->h, W, T, (int)W, sp.x_ff, sp.x_experts, sp.x_top, L.T(IFA_LT_X_UP).data, L.T(IFA_LT_X_DOWN).data, n->moe_idx,
+                                   n->moe_wgt, c.ops32, n->moe_ws, n->moe_ws_bytes, n->x, W, 1, s);
+}
+
 // the layers of one step over T rows / nseq sequences whose tables are already on the device; leaves the residual in n->x
 int run_layers(ifa_model *m, size_t T, int nseq)
 {
@@ -463,25 +547,42 @@ int run_layers(ifa_model *m, size_t T, int nseq)
     } else if (c.stem == 2) {
         if ((rc = ifa_embed_pair_f32(n->embd.data, c.vocab, c.width, c.bigram_buckets > 0 ? n->bigram.data : nullptr, c.bigram_buckets, c.bigram_mul_prev, c.bigram_mul_cur,
                                      n->tokens_dev, n->seqs_dev, n->row_seq_dev, T, slots, n->o_prev, n->x, s))) return rc;
+    } else if (c.stem == 3) {
+        if ((rc = ifa_embed_pair_scaled_f32(n->embd.data, c.vocab, c.width, c.embed_scale != 0.0f ? c.embed_scale : 1.0f, c.bigram_buckets > 0 ? n->bigram.data : nullptr,
+                                            c.bigram_buckets, c.bigram_mul_prev, c.bigram_mul_cur, n->tokens_dev, n->seqs_dev, n->row_seq_dev, T, slots, n->o_prev, n->x,
+                                            n->x0, s))) return rc;
     } else if ((rc = ifa_embed_sinpos_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, n->pos_dev, T, c.pos_base, n->x, s))) return rc;
     bool h_ready = false;
-    for (size_t li = 0; li < n->layers.size(); li++) {
+    for (size_t ri = 0; ri < n->runs.size(); ri++) {
+        const size_t li = (size_t)n->runs[ri].first;
+        const int pass = n->runs[ri].second;
         LLayer &L = n->layers[li];
         const ifa_layer_spec &sp = L.spec;
+        const LLayer *next_layer = ri + 1 < n->runs.size() ? &n->layers[(size_t)n->runs[ri + 1].first] : nullptr;
+        // a pass of the looped group starts from x (+ the embedding output, from the second pass on) + the pass's own vector
+        if (c.loop_times > 0 && (int)li == c.loop_start && c.loop_start < c.loop_stop
+            && (rc = ifa_add_rows_vec_f32(n->x, W, T, W, pass > 0 ? n->x0 : nullptr, W, (const bf16_t *)n->loop_step.data + (size_t)pass * W, s))) return rc;
+        if (sp.block == IFA_BLOCK_PRENORM) {
+            if ((rc = run_prenorm_layer(m, L, T, nseq, pass))) return rc;
+            h_ready = false;
+            if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
+                IFA_HIP_CHECK(hipMemcpyAsync(n->taps + ri * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
+            continue;
+        }
         if (sp.block == IFA_BLOCK_POSTNORM) {
             bool next_ready = false;
-            if ((rc = run_postnorm_layer(m, L, li, T, nseq, h_ready, li + 1 < n->layers.size() ? &n->layers[li + 1] : nullptr, &next_ready))) return rc;
+            if ((rc = run_postnorm_layer(m, L, li, T, nseq, h_ready, next_layer, &next_ready))) return rc;
             h_ready = next_ready;
             if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
-                IFA_HIP_CHECK(hipMemcpyAsync(n->taps + li * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
+                IFA_HIP_CHECK(hipMemcpyAsync(n->taps + ri * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
             continue;
         }
         if (sp.block == IFA_BLOCK_SANDWICH) {
             bool next_ready = false;
-            if ((rc = run_sandwich_layer(m, L, T, nseq, h_ready, li + 1 < n->layers.size() ? &n->layers[li + 1] : nullptr, &next_ready))) return rc;
+            if ((rc = run_sandwich_layer(m, L, T, nseq, h_ready, next_layer, &next_ready))) return rc;
             h_ready = next_ready;
             if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
-                IFA_HIP_CHECK(hipMemcpyAsync(n->taps + li * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
+                IFA_HIP_CHECK(hipMemcpyAsync(n->taps + ri * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
             continue;
         }
         const bf16_t *ls1 = (const bf16_t *)L.T(IFA_LT_LS1).data;
@@ -535,18 +636,21 @@ int run_layers(ifa_model *m, size_t T, int nseq)
             }
         }
         if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
-            IFA_HIP_CHECK(hipMemcpyAsync(n->taps + li * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
+            IFA_HIP_CHECK(hipMemcpyAsync(n->taps + ri * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
     }
     return IFA_OK;
 }
 
-// the norm in front of lm_head: layer norm without bias, (stem 1) the grouped RMS norm, or (stem 2) the RMS norm with weight (1 + w)
+float logit_scale_of(const LayeredNet *n) { return n->cfg.stem == 3 && n->cfg.logit_scale != 0.0f ? n->cfg.logit_scale : 1.0f; }
+
+// the norm in front of lm_head: (stem 3) the Dynamic Tanh norm, layer norm without bias, (stem 1) the grouped RMS norm, or (stem 2) the RMS norm with weight (1 + w)
 int out_norm_rows(ifa_model *m, const float *src, size_t rows, float *dst)
 {
     LayeredNet *n = m->lay;
     const size_t W = (size_t)n->cfg.width;
     if (n->cfg.stem == 1) return ifa_group_rmsnorm_f32(src, W, rows, W, n->cfg.norm_groups, n->out_norm.data, n->cfg.eps, 0, dst, W, (ifa_stream)m->stream);
     if (n->cfg.stem == 2) return ifa_rmsnorm_offset_f32(src, W, rows, W, n->out_norm.data, 1.0f, n->cfg.eps, 0, dst, W, (ifa_stream)m->stream);
+    if (n->cfg.stem == 3) return ifa_dyt_f32(src, W, rows, W, n->out_norm_alpha.data, n->out_norm.data, n->out_norm_b.data, dst, W, (ifa_stream)m->stream);
     return ifa_layernorm_f32(1, src, W, rows, W, n->out_norm.data, n->cfg.eps, dst, W, (ifa_stream)m->stream);
 }
 
@@ -563,7 +667,7 @@ int run_head(ifa_model *m, size_t r0, size_t nr)
         return IFA_OK;
     }
     if ((rc = out_norm_rows(m, n->x + r0 * W, nr, n->h))) return rc;
-    if ((rc = linear(m, (const bf16_t *)n->lm_head.data, V, W, n->h, W, nr, nullptr, nullptr, 1.0f, 0, n->logits, V))) return rc;
+    if ((rc = linear(m, (const bf16_t *)n->lm_head.data, V, W, n->h, W, nr, nullptr, nullptr, logit_scale_of(n), 0, n->logits, V))) return rc;
     if (n->cfg.logit_softcap > 0.0f && (rc = ifa_softcap_f32(n->logits, nr * V, n->cfg.logit_softcap, (ifa_stream)m->stream))) return rc;
     n->logits_rows = nr;
     return IFA_OK;
@@ -583,9 +687,11 @@ int lay_destroy(ifa_model *m)
     drop_step_graph(n);
     for (LLayer &L : n->layers) {
         for (LTensor &t : L.t) lay_free(t.data);
-        lay_free(L.w_in); lay_free(L.b_in); lay_free(L.w_conv); lay_free(L.bucket_of); lay_free(L.freq); lay_free(L.w_in2); lay_free(L.b_in2);
+        lay_free(L.w_in); lay_free(L.b_in); lay_free(L.w_conv); lay_free(L.bucket_of); lay_free(L.freq); lay_free(L.w_in2); lay_free(L.b_in2); lay_free(L.freq_v);
     }
     lay_free(n->embd.data); lay_free(n->out_norm.data); lay_free(n->lm_head.data); lay_free(n->embd_norm.data); lay_free(n->bigram.data);
+    lay_free(n->out_norm_b.data); lay_free(n->out_norm_alpha.data); lay_free(n->loop_step.data);
+    lay_free(n->x0); lay_free(n->cg_decay); lay_free(n->cg_unit); lay_free(n->cg_rem);
     lay_free(n->m4); lay_free(n->m5); lay_free(n->stack); lay_free(n->moe_wgt); lay_free(n->moe_idx); lay_free(n->moe_ws); lay_free(n->kx); lay_free(n->vx);
     for (float *p : n->slot_ptr) lay_free(p);
     lay_free(n->slot_base_dev);
@@ -619,14 +725,18 @@ int lay_finalize(ifa_model *m)
     const size_t W = (size_t)n->cfg.width;
     IFA_REQUIRE(n->embd.present() && n->out_norm.present() && n->lm_head.present(), "layer-list worker: embedding, final norm or lm_head is missing");
     IFA_REQUIRE(n->cfg.stem != 1 || n->embd_norm.present(), "layer-list worker: the norm behind the embedding is missing");
-    IFA_REQUIRE(n->cfg.stem != 2 || n->cfg.bigram_buckets <= 0 || n->bigram.present(), "layer-list worker: the token-pair embedding is missing");
+    IFA_REQUIRE((n->cfg.stem != 2 && n->cfg.stem != 3) || n->cfg.bigram_buckets <= 0 || n->bigram.present(), "layer-list worker: the token-pair embedding is missing");
+    IFA_REQUIRE(n->cfg.stem != 3 || (n->out_norm_b.present() && n->out_norm_alpha.present()), "layer-list worker: bias or scalar of the final norm is missing");
+    const bool looped = n->cfg.loop_times > 0 && n->cfg.loop_start < n->cfg.loop_stop;
+    IFA_REQUIRE(!looped || n->loop_step.present(), "layer-list worker: the vectors of the looped group's passes are missing");
     size_t off = 0;
-    if (n->cfg.stem == 2) { n->o_prev = off; off += 4; }
+    if (n->cfg.stem == 2 || n->cfg.stem == 3) { n->o_prev = off; off += 4; }
     n->n_in_max = n->mix_max = n->ffn_max = n->heads_max = 4;
     for (size_t li = 0; li < n->layers.size(); li++) {
         LLayer &L = n->layers[li];
         const ifa_layer_spec &sp = L.spec;
         if (L.w_in) continue;          // finalized before
+        const size_t off_layer = off;
         for (int id = IFA_LT_NORM1; id < IFA_LT_END; id++) {
             size_t r, c; bool vec;
             if (expected_shape(n, sp, (int)li, id, r, c, vec)) IFA_REQUIRE(L.T(id).present(), "layer-list worker: tensor %d of layer %zu is missing", id, li);
@@ -681,8 +791,26 @@ int lay_finalize(ifa_model *m)
             const int half = sp.a_rot_dims / 2;
             std::vector<double> fr((size_t)std::max(half, 1), 0.0);
             for (int i = 0; i < half; i++) fr[(size_t)i] = std::pow((double)sp.a_rot_base, -2.0 * i / (double)sp.a_rot_dims);
+            if (sp.a_rot_scale_factor > 0.0f) {
+                // by wavelength: short waves keep their frequency, long ones are slowed by the factor, a linear blend between
+                const double factor = sp.a_rot_scale_factor, lo = sp.a_rot_scale_low, hi = sp.a_rot_scale_high, orig = sp.a_rot_scale_original, two_pi = 6.283185307179586476925;
+                for (int i = 0; i < half; i++) {
+                    const double f = fr[(size_t)i], wl = two_pi / f;
+                    if (wl < orig / hi) continue;
+                    if (wl > orig / lo) { fr[(size_t)i] = f / factor; continue; }
+                    const double sm = (orig / wl - lo) / (hi - lo);
+                    fr[(size_t)i] = (1.0 - sm) * f / factor + sm * f;
+                }
+            }
             IFA_HIP_CHECK(hipMalloc((void **)&L.freq, fr.size() * 8));
             IFA_HIP_CHECK(hipMemcpy(L.freq, fr.data(), fr.size() * 8, hipMemcpyHostToDevice));
+            if (sp.a_vrot) {      // the values turn over their whole head with the plain frequencies
+                const int vh = sp.a_vdim / 2;
+                std::vector<double> fv((size_t)std::max(vh, 1), 0.0);
+                for (int i = 0; i < vh; i++) fv[(size_t)i] = std::pow((double)sp.a_rot_base, -2.0 * i / (double)sp.a_vdim);
+                IFA_HIP_CHECK(hipMalloc((void **)&L.freq_v, fv.size() * 8));
+                IFA_HIP_CHECK(hipMemcpy(L.freq_v, fv.data(), fv.size() * 8, hipMemcpyHostToDevice));
+            }
             if (own) {
                 L.o_k = off; off += align4((size_t)n->cfg.max_ctx * sp.a_kv_heads * sp.a_dim);
                 L.o_v = off; off += align4((size_t)n->cfg.max_ctx * sp.a_kv_heads * sp.a_vdim);
@@ -691,6 +819,13 @@ int lay_finalize(ifa_model *m)
             // the second product and the sizes of the feed-forward's buffers
             std::vector<bf16_t> w2, b2;
             size_t dummy;
+            if (sp.block == IFA_BLOCK_PRENORM) {      // (the router stays a product of its own: its choice takes it in for steps of a few rows)
+                if (has_moe(sp)) {
+                    n->mix_max = std::max(n->mix_max, (size_t)sp.x_experts);
+                    n->top_max = std::max(n->top_max, (size_t)sp.x_top);
+                    n->any_moe = true;
+                }
+            } else
             if (has_moe(sp)) {
                 if ((rc = cat_rows(w2, b2, L.T(IFA_LT_X_ROUTER), sp.x_route == 1 ? &L.T(IFA_LT_X_ROUTER_B) : nullptr, W, L.c2_router, m->stream))) return rc;
                 if (sp.x_shared_ff > 0) {
@@ -714,6 +849,19 @@ int lay_finalize(ifa_model *m)
                 IFA_HIP_CHECK(hipMemcpy(L.w_in2, w2.data(), w2.size() * 2, hipMemcpyHostToDevice));
                 IFA_HIP_CHECK(hipMemcpy(L.b_in2, b2.data(), b2.size() * 2, hipMemcpyHostToDevice));
                 n->n_in_max = std::max(n->n_in_max, L.n_in2);
+            }
+        } else if (sp.mixer == IFA_MIX_CHAN_DELTA) {
+            if ((rc = cat_rows(w, b, L.T(IFA_LT_C_R), nullptr, W, L.c_cr, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_C_K), nullptr, W, L.c_ck, m->stream))
+                || (rc = cat_rows(w, b, L.T(IFA_LT_C_V), nullptr, W, L.c_cv, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_C_G), nullptr, W, L.c_cg, m->stream))
+                || (rc = cat_rows(w, b, L.T(IFA_LT_C_A), &L.T(IFA_LT_C_A_B), W, L.c_ca, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_C_W1), nullptr, W, L.c_cw, m->stream))) return rc;
+            const size_t CH = (size_t)sp.c_heads * sp.c_dim;
+            L.o_rec = off; off += align4((size_t)sp.c_heads * sp.c_dim * sp.c_dim);
+            n->mix_max = std::max({n->mix_max, CH, W});
+            n->chan_max = std::max(n->chan_max, CH);
+            if (has_moe(sp)) {
+                n->mix_max = std::max(n->mix_max, (size_t)sp.x_experts);
+                n->top_max = std::max(n->top_max, (size_t)sp.x_top);
+                n->any_moe = true;
             }
         } else if (sp.mixer == IFA_MIX_WINDOW_LINEAR) {
             if ((rc = cat_rows(w, b, L.T(IFA_LT_A_Q), nullptr, W, L.c_aq, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_A_K), nullptr, W, L.c_ak, m->stream))
@@ -746,6 +894,11 @@ int lay_finalize(ifa_model *m)
             n->mix_max = std::max({n->mix_max, (size_t)L.conv_ch, DV});
             n->heads_max = std::max(n->heads_max, (size_t)sp.d_heads);
         }
+        // a layer of a looped group: its part of the arena once per pass
+        if (looped && (int)li >= n->cfg.loop_start && (int)li < n->cfg.loop_stop && n->cfg.loop_times > 1) {
+            L.pass_stride = off - off_layer;
+            off += (size_t)(n->cfg.loop_times - 1) * L.pass_stride;
+        }
         if (sp.ffn > 0 && sp.block != IFA_BLOCK_SANDWICH) {
             size_t up_off;
             if ((rc = cat_rows(w, b, L.T(IFA_LT_FFN_GATE), &L.T(IFA_LT_FFN_GATE_B), W, L.c_fg, m->stream))
@@ -763,7 +916,8 @@ int lay_finalize(ifa_model *m)
         // the separate copies of what the fused product now holds are no longer needed
         for (int id : {IFA_LT_A_Q, IFA_LT_A_K, IFA_LT_L_Q, IFA_LT_L_K, IFA_LT_L_V, IFA_LT_L_G, IFA_LT_D_Q, IFA_LT_D_K, IFA_LT_D_V, IFA_LT_D_B, IFA_LT_D_A,
                        IFA_LT_D_G, IFA_LT_FFN_GATE, IFA_LT_FFN_UP, IFA_LT_M_Q, IFA_LT_M_DQ, IFA_LT_M_DKV, IFA_LT_M_G, IFA_LT_A_V, IFA_LT_A_Q_B, IFA_LT_A_K_B,
-                       IFA_LT_A_V_B, IFA_LT_X_ROUTER_B, IFA_LT_X_SH_GATE, IFA_LT_X_SH_UP, IFA_LT_X_SH_SG}) {
+                       IFA_LT_A_V_B, IFA_LT_X_ROUTER_B, IFA_LT_X_SH_GATE, IFA_LT_X_SH_UP, IFA_LT_X_SH_SG, IFA_LT_C_R, IFA_LT_C_K, IFA_LT_C_V, IFA_LT_C_G, IFA_LT_C_A,
+                       IFA_LT_C_A_B, IFA_LT_C_W1}) {
             LTensor &t = L.T(id);
             if (t.data) { lay_free(t.data); t.data = nullptr; }
         }
@@ -777,6 +931,17 @@ int lay_finalize(ifa_model *m)
             else if (L.spec.mixer == IFA_MIX_LATENT) per_row = std::max(per_row, (size_t)L.spec.m_heads * 16 * ((size_t)L.spec.m_kv_rank + 2) * 4);
         n->attn_ws_bytes = per_row * 64;
         if (n->attn_ws_bytes) IFA_HIP_CHECK(hipMalloc((void **)&n->attn_ws, n->attn_ws_bytes));
+    }
+    // the stack as it is walked: the layers before the looped group, the group once per pass, the layers behind it
+    n->runs.clear();
+    for (int li = 0; li < (int)n->layers.size(); li++) {
+        if (looped && li == n->cfg.loop_start) {
+            for (int t = 0; t < n->cfg.loop_times; t++)
+                for (int lj = n->cfg.loop_start; lj < n->cfg.loop_stop; lj++) n->runs.push_back({lj, t});
+            li = n->cfg.loop_stop - 1;
+            continue;
+        }
+        n->runs.push_back({li, 0});
     }
     if (!n->slot_base_dev) {
         n->arena_floats = off;
@@ -840,9 +1005,10 @@ int lay_get_buffer(ifa_model *m, const char *name, int layer, void **dptr, size_
     size_t b = 0; void *p = nullptr;
     if (!strcmp(name, "logits")) { p = n->logits; b = n->logits_rows * (size_t)n->cfg.vocab * 4; }
     else if (!strcmp(name, "x")) { p = n->x; b = n->scratch_rows * (size_t)n->cfg.width * 4; }
-    else if (!strcmp(name, "layer_taps")) {      // [layers][taps_rows][width] fp32: the residual after every layer of the last step (option tap_layers)
+    else if (!strcmp(name, "layer_taps")) {      // [layer runs][taps_rows][width] fp32: the residual after every layer run of the last step (option tap_layers;
+                                                 // a layer of a looped group counts once per pass)
         IFA_REQUIRE(n->taps, "ifa_model_get_buffer: no taps (set option tap_layers before the step)");
-        IFA_REQUIRE(layer >= 0 && layer < (int)n->layers.size(), "ifa_model_get_buffer: layer %d", layer);
+        IFA_REQUIRE(layer >= 0 && layer < (int)n->runs.size(), "ifa_model_get_buffer: layer run %d", layer);
         p = n->taps + (size_t)layer * n->taps_rows * n->cfg.width; b = n->taps_rows * (size_t)n->cfg.width * 4;
     } else if (!strcmp(name, "slot")) {          // the arena of slot `layer`
         IFA_REQUIRE(layer >= 0 && layer < n->n_slots, "ifa_model_get_buffer: slot %d", layer);
@@ -887,7 +1053,7 @@ int ensure_taps(ifa_model *m, size_t T)
     if (!n->opt_tap_layers || T <= n->taps_rows) return IFA_OK;
     IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
     lay_free(n->taps); n->taps = nullptr;
-    IFA_HIP_CHECK(hipMalloc((void **)&n->taps, n->layers.size() * T * (size_t)n->cfg.width * 4));
+    IFA_HIP_CHECK(hipMalloc((void **)&n->taps, std::max(n->runs.size(), n->layers.size()) * T * (size_t)n->cfg.width * 4));
     n->taps_rows = T;
     return IFA_OK;
 }
@@ -943,7 +1109,7 @@ int lay_step(ifa_model *m, int nseq, const int *tokens_host, const int *lens, co
         // the sequences' last rows, normed one by one into consecutive rows of h, then one product
         for (int q = 0; q < nseq; q++)
             if ((rc = out_norm_rows(m, n->x + (size_t)last[(size_t)q] * W, 1, n->h + (size_t)q * W))) return rc;
-        if ((rc = linear(m, (const bf16_t *)n->lm_head.data, V, W, n->h, W, (size_t)nseq, nullptr, nullptr, 1.0f, 0, n->logits, V))) return rc;
+        if ((rc = linear(m, (const bf16_t *)n->lm_head.data, V, W, n->h, W, (size_t)nseq, nullptr, nullptr, logit_scale_of(n), 0, n->logits, V))) return rc;
         if (n->cfg.logit_softcap > 0.0f && (rc = ifa_softcap_f32(n->logits, (size_t)nseq * V, n->cfg.logit_softcap, s))) return rc;
         n->logits_rows = (size_t)nseq;
         if ((rc = ifa_argmax_rows_f32(n->logits, V, V, (size_t)nseq, n->excl_dev, n->next_dev, s))) return rc;
@@ -1070,9 +1236,24 @@ int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec
                 IFA_REQUIRE(o.mixer == IFA_MIX_ROTARY && o.a_kv_layer == 0 && o.a_kv_heads == s.a_kv_heads && o.a_dim == s.a_dim && o.a_vdim == s.a_vdim,
                             "ifa_model_create_layered: layer %d: layer %d has no keys and values of its own in this layer's shape", l, s.a_kv_layer - 1);
             }
+            IFA_REQUIRE(s.a_sink >= 0 && s.a_sink <= 2 && (s.a_rot_scale_factor == 0.0f || (s.a_rot_scale_factor > 0.0f && s.a_rot_scale_original > 0.0f
+                        && s.a_rot_scale_low > 0.0f && s.a_rot_scale_high > s.a_rot_scale_low)) && (!s.a_vrot || (s.a_vdim % 2 == 0 && s.a_rot_base > 1.0f)),
+                        "ifa_model_create_layered: layer %d: bad sink, frequency scaling or rotated values of an odd size", l);
+        } else if (s.mixer == IFA_MIX_CHAN_DELTA) {
+            IFA_REQUIRE(s.c_heads > 0 && s.c_dim > 0 && s.c_dim <= 256 && s.c_rank >= 1 && s.c_rank <= 8192 && s.c_decay_mult > 0.0f && s.c_l2_eps >= 0.0f,
+                        "ifa_model_create_layered: layer %d: bad sizes of the generalized delta rule", l);
         } else return ifa_fail(IFA_ERR_ARG, "ifa_model_create_layered: layer %d: unknown mixer %d", l, s.mixer);
-        IFA_REQUIRE((s.block == IFA_BLOCK_POSTNORM) == (s.mixer == IFA_MIX_LATENT) && (s.block == IFA_BLOCK_SANDWICH) == (s.mixer == IFA_MIX_ROTARY),
-                    "ifa_model_create_layered: layer %d: mixer %d is not wired for block kind %d", l, s.mixer, s.block);
+        const bool wired = s.mixer == IFA_MIX_LATENT ? s.block == IFA_BLOCK_POSTNORM
+                           : s.mixer == IFA_MIX_ROTARY ? (s.block == IFA_BLOCK_SANDWICH || s.block == IFA_BLOCK_PRENORM)
+                           : s.mixer == IFA_MIX_CHAN_DELTA ? s.block == IFA_BLOCK_PRENORM : s.block == IFA_BLOCK_PARALLEL;
+        IFA_REQUIRE(wired, "ifa_model_create_layered: layer %d: mixer %d is not wired for block kind %d", l, s.mixer, s.block);
+        if (s.block == IFA_BLOCK_PRENORM) {
+            IFA_REQUIRE(s.ffn == 0 && s.a_kv_layer == 0, "ifa_model_create_layered: layer %d: this wiring takes a mixture of experts or no feed-forward, and keys of its own", l);
+            if (s.ffn_kind == IFA_FFN_MOE && s.x_experts + s.x_identity > 0)
+                IFA_REQUIRE(s.x_identity == 0 && s.x_gated == 1 && s.x_route == 0 && s.x_shared_ff == 0 && s.x_experts >= 1 && s.x_experts <= 4096 && s.x_top >= 1
+                            && s.x_top <= s.x_experts && s.x_ff > 0 && (s.x_score == 0 || s.x_score == 1) && (s.x_glu == 0 || (s.x_glu == 3 && s.x_limit > 0.0f)),
+                            "ifa_model_create_layered: layer %d: bad mixture-of-experts sizes", l);
+        } else
         if (s.block == IFA_BLOCK_SANDWICH) {
             if (s.ffn_kind == IFA_FFN_MOE && s.x_experts + s.x_identity > 0)
                 IFA_REQUIRE(s.ffn == 0 && s.x_identity == 0 && s.x_gated == 1 && s.x_route == 1 && s.x_experts >= 1 && s.x_experts <= 4096 && s.x_top >= 1 && s.x_top <= s.x_experts
@@ -1088,7 +1269,14 @@ int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec
         } else IFA_REQUIRE(s.ffn_kind == IFA_FFN_GATED, "ifa_model_create_layered: layer %d: this wiring takes the gated feed-forward with biases", l);
     }
     IFA_REQUIRE(cfg->stem == 0 || (cfg->stem == 1 && cfg->norm_groups >= 1 && cfg->width % cfg->norm_groups == 0)
-                || (cfg->stem == 2 && cfg->bigram_buckets >= 0 && cfg->bigram_buckets < (1 << 30)), "ifa_model_create_layered: bad stem");
+                || ((cfg->stem == 2 || cfg->stem == 3) && cfg->bigram_buckets >= 0 && cfg->bigram_buckets < (1 << 30)), "ifa_model_create_layered: bad stem");
+    if (cfg->loop_times > 0 && cfg->loop_start < cfg->loop_stop) {
+        IFA_REQUIRE(cfg->loop_start >= 0 && cfg->loop_stop <= cfg->n_layers && cfg->loop_times <= 1024, "ifa_model_create_layered: looped group [%d, %d) x %d of %d layers",
+                    cfg->loop_start, cfg->loop_stop, cfg->loop_times, cfg->n_layers);
+        for (int l = cfg->loop_start; l < cfg->loop_stop; l++)
+            IFA_REQUIRE(layers[l].block == IFA_BLOCK_PRENORM, "ifa_model_create_layered: layer %d of the looped group is not wired with norms in front of its sub-layers", l);
+        IFA_REQUIRE(cfg->loop_times == 1 || cfg->stem == 3, "ifa_model_create_layered: a looped group of several passes needs the stem that keeps the embedding output");
+    }
     IFA_HIP_CHECK(hipSetDevice(cfg->device));
     ifa_model *m = new ifa_model();
     memset(&m->cfg, 0, sizeof(m->cfg));
@@ -1121,7 +1309,10 @@ int ifa_model_set_tensor_host(ifa_model *m, int layer, int tensor_id, int dtype,
         else if (tensor_id == IFA_T_LM_HEAD) { t = &n->lm_head; er = V; ec = W; }
         else if (tensor_id == IFA_T_OUT_NORM) { t = &n->out_norm; er = 1; ec = W; vec = true; }
         else if (tensor_id == IFA_T_EMBD_NORM) { t = &n->embd_norm; er = 1; ec = W; vec = true; }
-        else if (tensor_id == IFA_T_BIGRAM && n->cfg.stem == 2 && n->cfg.bigram_buckets > 0) { t = &n->bigram; er = (size_t)n->cfg.bigram_buckets + 1; ec = W; }
+        else if (tensor_id == IFA_T_BIGRAM && (n->cfg.stem == 2 || n->cfg.stem == 3) && n->cfg.bigram_buckets > 0) { t = &n->bigram; er = (size_t)n->cfg.bigram_buckets + 1; ec = W; }
+        else if (tensor_id == IFA_T_OUT_NORM_B && n->cfg.stem == 3) { t = &n->out_norm_b; er = 1; ec = W; vec = true; }
+        else if (tensor_id == IFA_T_OUT_NORM_ALPHA && n->cfg.stem == 3) { t = &n->out_norm_alpha; er = 1; ec = 1; vec = true; }
+        else if (tensor_id == IFA_T_LOOP_STEP && n->cfg.loop_times > 0) { t = &n->loop_step; er = (size_t)n->cfg.loop_times; ec = W; }
         else return ifa_fail(IFA_ERR_ARG, "ifa_model_set_tensor_host: global tensor id %d", tensor_id);
     } else {
         IFA_REQUIRE(layer < (int)n->layers.size() && tensor_id >= IFA_LT_NORM1 && tensor_id < IFA_LT_END, "ifa_model_set_tensor_host: layer %d / tensor id %d", layer, tensor_id);

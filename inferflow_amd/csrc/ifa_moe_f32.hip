@@ -23,20 +23,25 @@ typedef uint32_t u32x4m __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 
 // one wave per row: softmax over n_all logits, then `top` passes of argmax over score + correction (lowest index on ties)
+// (score_kind 1: the scores are the sigmoids of the logits instead of their softmax)
 __global__ void __launch_bounds__(64) k_moe_route(const float *__restrict__ logits, size_t ld, int n_all, int top, const bf16_t *__restrict__ corr,
-                                                  int *__restrict__ idx, float *__restrict__ wgt)
+                                                  int *__restrict__ idx, float *__restrict__ wgt, int score_kind)
 {
     extern __shared__ float sc[];          // [n_all] scores, [n_all] choice scores
     float *ch = sc + n_all;
     const int t = blockIdx.x, lane = threadIdx.x;
     const float *z = logits + (size_t)t * ld;
-    float mx = -INFINITY;
-    for (int e = lane; e < n_all; e += 64) mx = fmaxf(mx, z[e]);
-    mx = wave_max(mx);
-    float sum = 0.0f;
-    for (int e = lane; e < n_all; e += 64) { const float p = expf(z[e] - mx); sc[e] = p; sum += p; }
-    sum = wave_sum(sum);
-    for (int e = lane; e < n_all; e += 64) { const float s = sc[e] / sum; sc[e] = s; ch[e] = s + (corr ? bf2f(corr[e]) : 0.0f); }
+    if (score_kind == 1) {
+        for (int e = lane; e < n_all; e += 64) { const float s = sigmoid_f(z[e]); sc[e] = s; ch[e] = s + (corr ? bf2f(corr[e]) : 0.0f); }
+    } else {
+        float mx = -INFINITY;
+        for (int e = lane; e < n_all; e += 64) mx = fmaxf(mx, z[e]);
+        mx = wave_max(mx);
+        float sum = 0.0f;
+        for (int e = lane; e < n_all; e += 64) { const float p = expf(z[e] - mx); sc[e] = p; sum += p; }
+        sum = wave_sum(sum);
+        for (int e = lane; e < n_all; e += 64) { const float s = sc[e] / sum; sc[e] = s; ch[e] = s + (corr ? bf2f(corr[e]) : 0.0f); }
+    }
     __syncthreads();
     for (int k = 0; k < top; k++) {
         float best = -INFINITY; int bi = 0x7FFFFFFF;
@@ -80,7 +85,7 @@ __global__ void __launch_bounds__(64) k_moe_route_top(const float *__restrict__ 
 // Steps of a few rows: the router's product and its choice in one launch.  A workgroup per row: the waves share out the router's outputs
 // (a dot of `width` each), then the scores and the `top` passes as in k_moe_route (wave 0; the other waves only keep the barriers).
 __global__ void __launch_bounds__(1024) k_moe_route_rows(const float *__restrict__ h, size_t ldh, int W, const bf16_t *__restrict__ router, int n_all, int top,
-                                                        const bf16_t *__restrict__ corr, int *__restrict__ idx, float *__restrict__ wgt, int vec)
+                                                        const bf16_t *__restrict__ corr, int *__restrict__ idx, float *__restrict__ wgt, int vec, int score_kind)
 {
     extern __shared__ float sc[];          // [n_all] logits, then scores; [n_all] choice scores
     float *ch = sc + n_all;
@@ -106,7 +111,9 @@ __global__ void __launch_bounds__(1024) k_moe_route_rows(const float *__restrict
         if (lane == 0) sc[e] = acc;
     }
     __syncthreads();
-    if (wave == 0) {
+    if (wave == 0 && score_kind == 1) {
+        for (int e = lane; e < n_all; e += 64) { const float sv = sigmoid_f(sc[e]); sc[e] = sv; ch[e] = sv + (corr ? bf2f(corr[e]) : 0.0f); }
+    } else if (wave == 0) {
         float mx = -INFINITY;
         for (int e = lane; e < n_all; e += 64) mx = fmaxf(mx, sc[e]);
         mx = wave_max(mx);
@@ -133,7 +140,7 @@ __global__ void __launch_bounds__(1024) k_moe_route_rows(const float *__restrict
 // grid (ff chunks, pairs): act[p][n] = gelu(W_up[e][n] . h[t]); a wave per n at a time.  Identity pairs do nothing.
 template <bool GATED>
 __global__ void __launch_bounds__(256) k_moe_up_rows(const float *__restrict__ h, size_t ldh, int W, int F, int experts, int top, const bf16_t *__restrict__ up,
-                                                     const int *__restrict__ idx, float *__restrict__ act, int vec)
+                                                     const int *__restrict__ idx, float *__restrict__ act, int vec, int glu_kind, float limit)
 {
     const int p = blockIdx.y, e = idx[p];
     if (e >= experts) return;
@@ -159,7 +166,10 @@ __global__ void __launch_bounds__(256) k_moe_up_rows(const float *__restrict__ h
                 for (int k = lane; k < W; k += 64) { ag = fmaf(hr[k], bf2f(wg[k]), ag); au = fmaf(hr[k], bf2f(wu[k]), au); }
             }
             ag = wave_sum(ag); au = wave_sum(au);
-            if (lane == 0) act[(size_t)p * F + n] = silu_exact(ag) * au;
+            if (lane == 0) {
+                if (glu_kind == 3) { const float g = fminf(ag, limit), u = fminf(fmaxf(au, -limit), limit); act[(size_t)p * F + n] = g * sigmoid_f(1.702f * g) * (u + 1.0f); }
+                else act[(size_t)p * F + n] = silu_exact(ag) * au;
+            }
         }
         return;
     }
@@ -294,25 +304,39 @@ size_t moe_tiles_max(size_t rows, int top, int experts) { return (rows * (size_t
 
 extern "C" {
 
+int ifa_moe_route_scores_f32(int score_kind, const void *logits_f32, size_t ld, size_t rows, int n_all, int top, const void *correction_bf16, int *idx_dev,
+                             void *wgt_f32, ifa_stream stream)
+{
+    IFA_REQUIRE(logits_f32 && idx_dev && wgt_f32, "ifa_moe_route_scores_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ld >= (size_t)n_all && (score_kind == 0 || score_kind == 1),
+                "ifa_moe_route_scores_f32: bad shape (%d router outputs, %d chosen, scores of kind %d)", n_all, top, score_kind);
+    hipLaunchKernelGGL(k_moe_route, dim3((unsigned)rows), dim3(64), (size_t)n_all * 8, ifa_s(stream), (const float *)logits_f32, ld, n_all, top,
+                       (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32, score_kind);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
 int ifa_moe_route_f32(const void *logits_f32, size_t ld, size_t rows, int n_all, int top, const void *correction_bf16, int *idx_dev, void *wgt_f32,
                       ifa_stream stream)
 {
-    IFA_REQUIRE(logits_f32 && idx_dev && wgt_f32, "ifa_moe_route_f32: null pointer");
-    IFA_REQUIRE(rows > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ld >= (size_t)n_all, "ifa_moe_route_f32: bad shape (%d router outputs, %d chosen)", n_all, top);
-    hipLaunchKernelGGL(k_moe_route, dim3((unsigned)rows), dim3(64), (size_t)n_all * 8, ifa_s(stream), (const float *)logits_f32, ld, n_all, top,
-                       (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32);
-    IFA_LAUNCH_CHECK();
-    return IFA_OK;
+    return ifa_moe_route_scores_f32(0, logits_f32, ld, rows, n_all, top, correction_bf16, idx_dev, wgt_f32, stream);
 }
 
 int ifa_moe_route_rows_f32(const void *h_f32, size_t ldh, size_t rows, int width, const void *router_bf16, int n_all, int top, const void *correction_bf16,
                            int *idx_dev, void *wgt_f32, ifa_stream stream)
 {
+    return ifa_moe_route_rows_scores_f32(0, h_f32, ldh, rows, width, router_bf16, n_all, top, correction_bf16, idx_dev, wgt_f32, stream);
+}
+
+int ifa_moe_route_rows_scores_f32(int score_kind, const void *h_f32, size_t ldh, size_t rows, int width, const void *router_bf16, int n_all, int top,
+                                  const void *correction_bf16, int *idx_dev, void *wgt_f32, ifa_stream stream)
+{
     IFA_REQUIRE(h_f32 && router_bf16 && idx_dev && wgt_f32, "ifa_moe_route_rows_f32: null pointer");
-    IFA_REQUIRE(rows > 0 && rows <= 64 && width > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ldh >= (size_t)width, "ifa_moe_route_rows_f32: bad shape");
+    IFA_REQUIRE(rows > 0 && rows <= 64 && width > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ldh >= (size_t)width && (score_kind == 0 || score_kind == 1),
+                "ifa_moe_route_rows_f32: bad shape");
     const int vec = (width % 8 == 0 && ldh % 4 == 0 && ((uintptr_t)h_f32 & 15) == 0 && ((uintptr_t)router_bf16 & 15) == 0) ? 1 : 0;
     hipLaunchKernelGGL(k_moe_route_rows, dim3((unsigned)rows), dim3(n_all > 8 ? 1024 : 256), (size_t)n_all * 8, ifa_s(stream), (const float *)h_f32, ldh, width,
-                       (const bf16_t *)router_bf16, n_all, top, (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32, vec);
+                       (const bf16_t *)router_bf16, n_all, top, (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32, vec, score_kind);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }
@@ -334,7 +358,7 @@ size_t ifa_moe_workspace_bytes(size_t rows, int top, int width, int ff, int expe
     return al16(pairs * ff * 4) + al16(pairs * width * 4) + 3 * al16(pairs * 4) + al16(moe_tiles_max(rows, top, experts) * 12) + 16;
 }
 
-static int moe_experts(const char *who, int gated, const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int identity, int top, int act,
+static int moe_experts(const char *who, int gated, int glu_kind, float limit, const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int identity, int top, int act,
                        const void *up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
                        void *y_f32, size_t ldy, int accumulate, ifa_stream stream)
 {
@@ -362,10 +386,10 @@ static int moe_experts(const char *who, int gated, const void *h_f32, size_t ldh
         const int vec_d = (ff % 8 == 0 && ((uintptr_t)down_bf16 & 15) == 0) ? 1 : 0;
         if (experts > 0 && gated)
             hipLaunchKernelGGL(k_moe_up_rows<true>, dim3(std::min(512u, ifa_cdiv((size_t)ff, 4)), (unsigned)pairs), dim3(256), 0, s, h, ldh, width, ff, experts, top,
-                               (const bf16_t *)up_bf16, idx_dev, actb, vec_u);
+                               (const bf16_t *)up_bf16, idx_dev, actb, vec_u, glu_kind, limit);
         else if (experts > 0)
             hipLaunchKernelGGL(k_moe_up_rows<false>, dim3(std::min(512u, ifa_cdiv((size_t)ff, 4)), (unsigned)pairs), dim3(256), 0, s, h, ldh, width, ff, experts, top,
-                               (const bf16_t *)up_bf16, idx_dev, actb, vec_u);
+                               (const bf16_t *)up_bf16, idx_dev, actb, vec_u, 0, 0.0f);
         hipLaunchKernelGGL(k_moe_down_rows, dim3(std::min(1024u, ifa_cdiv((size_t)width, 4)), (unsigned)rows), dim3(256), 0, s, h, ldh, width, ff, experts, top,
                            (const bf16_t *)down_bf16, idx_dev, (const float *)wgt_f32, actb, accumulate ? 1 : 0, (float *)y_f32, ldy, vec_d);
         IFA_LAUNCH_CHECK();
@@ -379,7 +403,7 @@ static int moe_experts(const char *who, int gated, const void *h_f32, size_t ldh
     int rc;
     if (gated) {
         if ((rc = ifa_linear_bf16w_grouped(up_bf16, (size_t)2 * ff, (size_t)width, experts, h_f32, ldh, a_rows, tile_map, n_tiles, max_tiles, nullptr, 0, ops32, gub, (size_t)2 * ff, stream))) return rc;
-        if ((rc = ifa_glu_f32(0, gub, (size_t)2 * ff, pairs, (size_t)ff, actb, (size_t)ff, stream))) return rc;
+        if ((rc = ifa_glu_ex_f32(glu_kind, limit, gub, (size_t)2 * ff, pairs, (size_t)ff, nullptr, 0, actb, (size_t)ff, stream))) return rc;
     } else
     if ((rc = ifa_linear_bf16w_grouped(up_bf16, (size_t)ff, (size_t)width, experts, h_f32, ldh, a_rows, tile_map, n_tiles, max_tiles, nullptr, 1, ops32, actb, (size_t)ff, stream))) return rc;
     if ((rc = ifa_linear_bf16w_grouped(down_bf16, (size_t)width, (size_t)ff, experts, actb, (size_t)ff, nullptr, tile_map, n_tiles, max_tiles, w_sorted, 0, ops32, yp, (size_t)width, stream))) return rc;
@@ -393,7 +417,7 @@ int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, i
                         const void *up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
                         void *y_f32, size_t ldy, int accumulate, ifa_stream stream)
 {
-    return moe_experts("ifa_moe_experts_f32", 0, h_f32, ldh, rows, width, ff, experts, identity, top, act, up_bf16, down_bf16, idx_dev, wgt_f32, ops32, ws, ws_bytes, y_f32,
+    return moe_experts("ifa_moe_experts_f32", 0, 0, 0.0f, h_f32, ldh, rows, width, ff, experts, identity, top, act, up_bf16, down_bf16, idx_dev, wgt_f32, ops32, ws, ws_bytes, y_f32,
                        ldy, accumulate, stream);
 }
 
@@ -402,8 +426,17 @@ int ifa_moe_experts_gated_f32(const void *h_f32, size_t ldh, size_t rows, int wi
                               int accumulate, ifa_stream stream)
 {
     IFA_REQUIRE(experts > 0, "ifa_moe_experts_gated_f32: no experts");
-    return moe_experts("ifa_moe_experts_gated_f32", 1, h_f32, ldh, rows, width, ff, experts, 0, top, 0, gate_up_bf16, down_bf16, idx_dev, wgt_f32, ops32, ws, ws_bytes,
+    return moe_experts("ifa_moe_experts_gated_f32", 1, 0, 0.0f, h_f32, ldh, rows, width, ff, experts, 0, top, 0, gate_up_bf16, down_bf16, idx_dev, wgt_f32, ops32, ws, ws_bytes,
                        y_f32, ldy, accumulate, stream);
+}
+
+int ifa_moe_experts_glu_f32(int glu_kind, float limit, const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int top,
+                            const void *gate_up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
+                            void *y_f32, size_t ldy, int accumulate, ifa_stream stream)
+{
+    IFA_REQUIRE(experts > 0 && (glu_kind == 0 || (glu_kind == 3 && limit > 0.0f)), "ifa_moe_experts_glu_f32: no experts, or gate kind %d (0, or 3 with a limit)", glu_kind);
+    return moe_experts("ifa_moe_experts_glu_f32", 1, glu_kind, limit, h_f32, ldh, rows, width, ff, experts, 0, top, 0, gate_up_bf16, down_bf16, idx_dev, wgt_f32, ops32, ws,
+                       ws_bytes, y_f32, ldy, accumulate, stream);
 }
 
 } // extern "C"

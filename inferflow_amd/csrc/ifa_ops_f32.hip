@@ -1,5 +1,6 @@
 // ifa_ops_f32.hip -- element-wise and row ops on 32-bit activations with bfloat16 parameters: embedding rows with a sinusoidal
 // position vector, layer / RMS norm, gated activations, greedy argmax, and the conversions the F16 interfaces need.
+#include <algorithm>
 #include "ifa_host.h"
 #include "ifa_f32_common.h"
 
@@ -81,7 +82,7 @@ __global__ void __launch_bounds__(256) k_group_rmsnorm(const float *__restrict__
 __global__ void __launch_bounds__(256) k_embed_pair(const bf16_t *__restrict__ embed, int vocab, int width, const bf16_t *__restrict__ pair, int buckets,
                                                     int mul_prev, int mul_cur, const int *__restrict__ tokens, const SeqDesc *__restrict__ seqs,
                                                     const int *__restrict__ row_seq, float *const *__restrict__ slot_base, size_t state_off,
-                                                    float *__restrict__ x)
+                                                    float *__restrict__ x, float embed_scale, float *__restrict__ x_copy)
 {
     const int t = blockIdx.x;
     const SeqDesc sd = seqs[row_seq[t]];
@@ -99,9 +100,46 @@ __global__ void __launch_bounds__(256) k_embed_pair(const bf16_t *__restrict__ e
     __syncthreads();      // (the read of the cell above is done in every thread before thread 0 rewrites it)
     if (t == sd.row0 && threadIdx.x == 0) *cell = tokens[sd.row0 + sd.n - 1];
     for (int c = threadIdx.x; c < width; c += blockDim.x) {
-        float v = bf2f(embed[(size_t)tok * width + c]);
+        float v = bf2f(embed[(size_t)tok * width + c]) * embed_scale;
         if (pair) v += bf2f(pair[(size_t)prow * width + c]);
         x[(size_t)t * width + c] = v;
+        if (x_copy) x_copy[(size_t)t * width + c] = v;
+    }
+}
+
+// Dynamic Tanh: y = tanh(alpha x) w + b, element by element (alpha: one bfloat16 value)
+__global__ void __launch_bounds__(256) k_dyt(const float *__restrict__ x, size_t ldx, int cols, const bf16_t *__restrict__ alpha, const bf16_t *__restrict__ w,
+                                             const bf16_t *__restrict__ b, float *__restrict__ y, size_t ldy)
+{
+    const float a = bf2f(alpha[0]);
+    const float *xr = x + (size_t)blockIdx.x * ldx;
+    float *yr = y + (size_t)blockIdx.x * ldy;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < cols; c += gridDim.y * blockDim.x) yr[c] = fmaf(tanhf(a * xr[c]), bf2f(w[c]), bf2f(b[c]));
+}
+
+// x += m, then h = tanh(alpha x) w + b: the residual update behind a sub-layer and the norm in front of the next one
+__global__ void __launch_bounds__(256) k_add_dyt(float *__restrict__ x, size_t ldx, int cols, const float *__restrict__ m, size_t ldm, const bf16_t *__restrict__ alpha,
+                                                 const bf16_t *__restrict__ w, const bf16_t *__restrict__ b, float *__restrict__ h, size_t ldh)
+{
+    const float a = w ? bf2f(alpha[0]) : 0.0f;
+    float *xr = x + (size_t)blockIdx.x * ldx;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < cols; c += gridDim.y * blockDim.x) {
+        float v = xr[c];
+        if (m) { v += m[(size_t)blockIdx.x * ldm + c]; xr[c] = v; }
+        if (w) h[(size_t)blockIdx.x * ldh + c] = fmaf(tanhf(a * v), bf2f(w[c]), bf2f(b[c]));
+    }
+}
+
+// x[t][c] += add[t][c] + vec[c] (either may be absent)
+__global__ void __launch_bounds__(256) k_add_rows_vec(float *__restrict__ x, size_t ldx, int cols, const float *__restrict__ add, size_t lda,
+                                                      const bf16_t *__restrict__ vec)
+{
+    float *xr = x + (size_t)blockIdx.x * ldx;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < cols; c += gridDim.y * blockDim.x) {
+        float v = xr[c];
+        if (add) v += add[(size_t)blockIdx.x * lda + c];
+        if (vec) v += bf2f(vec[c]);
+        xr[c] = v;
     }
 }
 
@@ -308,7 +346,56 @@ int ifa_embed_pair_f32(const void *embed_bf16, int vocab, int width, const void 
     IFA_REQUIRE(embed_bf16 && tokens_dev && seqs_dev && row_seq_dev && slot_base_dev && x_f32, "ifa_embed_pair_f32: null pointer");
     IFA_REQUIRE(vocab > 0 && width > 0 && rows > 0 && (!pair_bf16 || buckets > 0), "ifa_embed_pair_f32: bad shape");
     hipLaunchKernelGGL(k_embed_pair, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (const bf16_t *)embed_bf16, vocab, width, (const bf16_t *)pair_bf16, buckets,
-                       mul_prev, mul_cur, tokens_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, state_off, (float *)x_f32);
+                       mul_prev, mul_cur, tokens_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, state_off, (float *)x_f32, 1.0f,
+                       (float *)nullptr);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_embed_pair_scaled_f32(const void *embed_bf16, int vocab, int width, float embed_scale, const void *pair_bf16, int buckets, int mul_prev, int mul_cur,
+                              const int *tokens_dev, const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t state_off,
+                              void *x_f32, void *x_copy_f32, ifa_stream stream)
+{
+    IFA_REQUIRE(embed_bf16 && tokens_dev && seqs_dev && row_seq_dev && slot_base_dev && x_f32, "ifa_embed_pair_scaled_f32: null pointer");
+    IFA_REQUIRE(vocab > 0 && width > 0 && rows > 0 && (!pair_bf16 || buckets > 0), "ifa_embed_pair_scaled_f32: bad shape");
+    hipLaunchKernelGGL(k_embed_pair, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (const bf16_t *)embed_bf16, vocab, width, (const bf16_t *)pair_bf16, buckets,
+                       mul_prev, mul_cur, tokens_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, state_off, (float *)x_f32, embed_scale,
+                       (float *)x_copy_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+static dim3 rows_grid(size_t rows, size_t cols) { return dim3((unsigned)rows, (unsigned)std::min<size_t>(16, (cols + 255) / 256)); }
+
+int ifa_dyt_f32(const void *x_f32, size_t ldx, size_t rows, size_t cols, const void *alpha_bf16, const void *w_bf16, const void *b_bf16, void *y_f32,
+                size_t ldy, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && alpha_bf16 && w_bf16 && b_bf16 && y_f32, "ifa_dyt_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && rows < (1u << 31) && cols > 0 && ldx >= cols && ldy >= cols, "ifa_dyt_f32: bad arguments");
+    hipLaunchKernelGGL(k_dyt, rows_grid(rows, cols), dim3(256), 0, ifa_s(stream), (const float *)x_f32, ldx, (int)cols, (const bf16_t *)alpha_bf16,
+                       (const bf16_t *)w_bf16, (const bf16_t *)b_bf16, (float *)y_f32, ldy);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_add_dyt_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *alpha_bf16, const void *w_bf16,
+                    const void *b_bf16, void *h_f32, size_t ldh, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && (!w_bf16 || (alpha_bf16 && b_bf16 && h_f32)), "ifa_add_dyt_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && rows < (1u << 31) && cols > 0 && ldx >= cols && (!m_f32 || ldm >= cols) && (!w_bf16 || ldh >= cols), "ifa_add_dyt_f32: bad arguments");
+    if (!m_f32 && !w_bf16) return IFA_OK;
+    hipLaunchKernelGGL(k_add_dyt, rows_grid(rows, cols), dim3(256), 0, ifa_s(stream), (float *)x_f32, ldx, (int)cols, (const float *)m_f32, ldm,
+                       (const bf16_t *)alpha_bf16, (const bf16_t *)w_bf16, (const bf16_t *)b_bf16, (float *)h_f32, ldh);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_add_rows_vec_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *add_f32, size_t lda, const void *vec_bf16, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && rows > 0 && rows < (1u << 31) && cols > 0 && ldx >= cols && (!add_f32 || lda >= cols), "ifa_add_rows_vec_f32: bad arguments");
+    if (!add_f32 && !vec_bf16) return IFA_OK;
+    hipLaunchKernelGGL(k_add_rows_vec, rows_grid(rows, cols), dim3(256), 0, ifa_s(stream), (float *)x_f32, ldx, (int)cols, (const float *)add_f32, lda,
+                       (const bf16_t *)vec_bf16);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -5,6 +5,8 @@
 //     (in_act = 1: q, k, v pass SiLU as they are read)
 //       kind 1  gated delta rule:                                 S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 //   * the gates of the delta rule (beta = sigmoid, g = exp(-exp(A_log) softplus(a + dt_bias)))
+//   * the generalized delta rule with a decay w and a removal rate per key channel: S <- diag(w) S - b (u^T S) + k v^T, o = S^T q
+//     (u the unit key, b = removal rate * u), and its gates
 //   * RMS norm over channel groups with a weight and an output gate (sigmoid or SiLU)
 // Everything that enters a recurrence is fp32; states live in fp32 in the slot arena of the worker (a table of one
 // base pointer per slot + an offset per layer).  A sequence that starts at position 0 starts from a zero state,
@@ -369,6 +371,186 @@ __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
     }
 }
 
+// ---- generalized delta rule with a decay and a removal rate per key channel:
+//   S <- diag(w_t) S - b_t (u_t^T S) + k_t v_t^T   (both terms read the old state),   o_t = S^T q_t
+// w (decay), u (unit key) and b (removal rate times unit key) come per row and key channel from k_chan_delta_gates.
+// one workgroup per row: the bottleneck's activations tanh(lr) in LDS, then a wave per head at a time:
+// decay = exp(-mult * sigmoid(w2[c] . tanh(lr) + w0[c])), u = k / sqrt(sum k^2 + l2_eps), b = sigmoid(a) * u
+__global__ void __launch_bounds__(256) k_chan_delta_gates(const float *__restrict__ lr, size_t ldl, int rank, const bf16_t *__restrict__ w2, const bf16_t *__restrict__ w0,
+                                                          float mult, const float *__restrict__ a, size_t lda, const float *__restrict__ k, size_t ldk, int H, int D,
+                                                          float l2_eps, float *__restrict__ decay, float *__restrict__ unit, float *__restrict__ removal)
+{
+    extern __shared__ float th[];          // [rank]
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    for (int i = threadIdx.x; i < rank; i += blockDim.x) th[i] = tanhf(lr[(size_t)t * ldl + i]);
+    __syncthreads();
+    const size_t HD = (size_t)H * D;
+    for (int h = wave; h < H; h += nw) {
+        const float *kr = k + (size_t)t * ldk + (size_t)h * D;
+        float s = 0.0f;
+        for (int c = lane; c < D; c += 64) s = fmaf(kr[c], kr[c], s);
+        const float rinv = 1.0f / sqrtf(wave_sum(s) + l2_eps);
+        for (int c = lane; c < D; c += 64) {
+            const size_t hc = (size_t)h * D + c;
+            const bf16_t *wr = w2 + hc * (size_t)rank;
+            float z0 = w0 ? bf2f(w0[hc]) : 0.0f, z1 = 0.0f;
+            int i = 0;
+            for (; i + 1 < rank; i += 2) { z0 = fmaf(bf2f(wr[i]), th[i], z0); z1 = fmaf(bf2f(wr[i + 1]), th[i + 1], z1); }
+            if (i < rank) z0 = fmaf(bf2f(wr[i]), th[i], z0);
+            const float u = kr[c] * rinv;
+            decay[(size_t)t * HD + hc] = expf(-mult * sigmoid_f(z0 + z1));
+            unit[(size_t)t * HD + hc] = u;
+            removal[(size_t)t * HD + hc] = sigmoid_f(a[(size_t)t * lda + hc]) * u;
+        }
+    }
+}
+
+struct ChanScanArgs {
+    const float *q, *k, *v; size_t ldq, ldk, ldv;
+    const float *w, *u, *b; size_t ldg;
+    int heads, dk, dv;
+    const SeqDesc *seqs; float *const *slot_base; size_t state_off;
+    float *out; size_t ldo;
+};
+
+// any dk <= 64 * SCAN_DKL: grid (sequences * heads, ceil(dv / 64)), one wave; a lane owns a column of S in LDS ([dk][64])
+__global__ void __launch_bounds__(64) k_state_scan_chan(ChanScanArgs P)
+{
+    extern __shared__ float sm[];
+    const int dk = P.dk;
+    float *S = sm, *qs = sm + (size_t)dk * 64, *ks = qs + dk, *ws = ks + dk, *us = ws + dk, *bs = us + dk;
+    const int seq = blockIdx.x / P.heads, h = blockIdx.x % P.heads;
+    const int lane = threadIdx.x, j = blockIdx.y * 64 + lane;
+    const bool live = j < P.dv;
+    const int jc = live ? j : P.dv - 1;
+    const SeqDesc sd = P.seqs[seq];
+    float *state = P.slot_base[sd.slot] + P.state_off + (size_t)h * dk * P.dv;
+    if (sd.pos0 > 0) for (int i = 0; i < dk; i++) S[i * 64 + lane] = state[(size_t)i * P.dv + jc];
+    else for (int i = 0; i < dk; i++) S[i * 64 + lane] = 0.0f;
+    float qr[SCAN_DKL], kr[SCAN_DKL], wr[SCAN_DKL], ur[SCAN_DKL], br[SCAN_DKL], vr = 0.0f;
+    auto request = [&](int t) {
+        const size_t row = (size_t)(sd.row0 + t);
+#pragma unroll
+        for (int e = 0; e < SCAN_DKL; e++) {
+            const int i = lane + 64 * e;
+            if (i < dk) {
+                const size_t hc = (size_t)h * dk + i;
+                qr[e] = P.q[row * P.ldq + hc]; kr[e] = P.k[row * P.ldk + hc];
+                wr[e] = P.w[row * P.ldg + hc]; ur[e] = P.u[row * P.ldg + hc]; br[e] = P.b[row * P.ldg + hc];
+            }
+        }
+        vr = P.v[row * P.ldv + (size_t)h * P.dv + jc];
+    };
+    if (sd.n > 0) request(0);
+    for (int t = 0; t < sd.n; t++) {
+        __syncthreads();          // the previous token's reads of the staged vectors are done
+#pragma unroll
+        for (int e = 0; e < SCAN_DKL; e++) { const int i = lane + 64 * e; if (i < dk) { qs[i] = qr[e]; ks[i] = kr[e]; ws[i] = wr[e]; us[i] = ur[e]; bs[i] = br[e]; } }
+        const float vt = vr;
+        __syncthreads();
+        if (t + 1 < sd.n) request(t + 1);
+        float sa = 0.0f, o = 0.0f;
+        for (int i = 0; i < dk; i++) sa = fmaf(us[i], S[i * 64 + lane], sa);
+        for (int i = 0; i < dk; i++) {
+            const float s = fmaf(ks[i], vt, fmaf(ws[i], S[i * 64 + lane], -bs[i] * sa));
+            S[i * 64 + lane] = s;
+            o = fmaf(s, qs[i], o);
+        }
+        if (live) P.out[(size_t)(sd.row0 + t) * P.ldo + (size_t)h * P.dv + j] = o;
+    }
+    if (live) for (int i = 0; i < dk; i++) state[(size_t)i * P.dv + j] = S[i * 64 + lane];
+}
+
+// key sizes 16 / 32 / 48 / 64 / 96 / 128: the state in registers, LPC lanes per column (as k_state_scan_reg), token groups of SCAN_TB staged in LDS
+template <int DK, int LPC>
+__global__ void __launch_bounds__(64) k_state_scan_chan_reg(ChanScanArgs P)
+{
+    constexpr int DKQ = DK / LPC, CPW = 64 / LPC;
+    __shared__ __attribute__((aligned(16))) float qs[2][SCAN_TB][DK], ks[2][SCAN_TB][DK], ws[2][SCAN_TB][DK], us[2][SCAN_TB][DK], bs[2][SCAN_TB][DK];
+    const int seq = blockIdx.x / P.heads, h = blockIdx.x % P.heads;
+    const int lane = threadIdx.x, rg = lane & (LPC - 1), j = blockIdx.y * CPW + lane / LPC;
+    const bool live = j < P.dv;
+    const int jc = live ? j : P.dv - 1;
+    const SeqDesc sd = P.seqs[seq];
+    float *state = P.slot_base[sd.slot] + P.state_off + ((size_t)h * DK + (size_t)rg * DKQ) * P.dv;
+    float S[DKQ];
+    if (sd.pos0 > 0) {
+#pragma unroll
+        for (int e = 0; e < DKQ; e++) S[e] = state[(size_t)e * P.dv + jc];
+    } else {
+#pragma unroll
+        for (int e = 0; e < DKQ; e++) S[e] = 0.0f;
+    }
+    constexpr int PER = SCAN_TB * DK / 64;
+    float qr[PER], kr[PER], wr[PER], ur[PER], br[PER], vnext[SCAN_TB], vcur[SCAN_TB];
+    auto request = [&](int t0) {
+#pragma unroll
+        for (int x = 0; x < PER; x++) {
+            const int e = lane + 64 * x, tt = e / DK, i = e % DK;
+            const size_t row = (size_t)(sd.row0 + min(t0 + tt, sd.n - 1)), hc = (size_t)h * DK + i;
+            qr[x] = P.q[row * P.ldq + hc]; kr[x] = P.k[row * P.ldk + hc];
+            wr[x] = P.w[row * P.ldg + hc]; ur[x] = P.u[row * P.ldg + hc]; br[x] = P.b[row * P.ldg + hc];
+        }
+#pragma unroll
+        for (int tt = 0; tt < SCAN_TB; tt++) {
+            const size_t row = (size_t)(sd.row0 + min(t0 + tt, sd.n - 1));
+            vnext[tt] = P.v[row * P.ldv + (size_t)h * P.dv + jc];
+        }
+    };
+    auto publish = [&](int buf) {
+#pragma unroll
+        for (int x = 0; x < PER; x++) {
+            const int e = lane + 64 * x, tt = e / DK, i = e % DK;
+            qs[buf][tt][i] = qr[x]; ks[buf][tt][i] = kr[x]; ws[buf][tt][i] = wr[x]; us[buf][tt][i] = ur[x]; bs[buf][tt][i] = br[x];
+        }
+#pragma unroll
+        for (int tt = 0; tt < SCAN_TB; tt++) vcur[tt] = vnext[tt];
+    };
+    if (sd.n > 0) { request(0); publish(0); }
+    __syncthreads();
+    for (int t0 = 0, buf = 0; t0 < sd.n; t0 += SCAN_TB, buf ^= 1) {
+        const bool more = t0 + SCAN_TB < sd.n;
+        if (more) request(t0 + SCAN_TB);
+        const int cnt = min(SCAN_TB, sd.n - t0);
+#pragma unroll
+        for (int tt = 0; tt < SCAN_TB; tt++) {
+            if (tt < cnt) {
+                const float vt = vcur[tt];
+                float kk[DKQ], qq[DKQ], ww[DKQ], uu[DKQ], bb[DKQ];
+#pragma unroll
+                for (int e4 = 0; e4 < DKQ; e4 += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4 *>(&ks[buf][tt][rg * DKQ + e4]), q4 = *reinterpret_cast<const float4 *>(&qs[buf][tt][rg * DKQ + e4]);
+                    const float4 w4 = *reinterpret_cast<const float4 *>(&ws[buf][tt][rg * DKQ + e4]), u4 = *reinterpret_cast<const float4 *>(&us[buf][tt][rg * DKQ + e4]);
+                    const float4 b4 = *reinterpret_cast<const float4 *>(&bs[buf][tt][rg * DKQ + e4]);
+                    kk[e4] = k4.x; kk[e4 + 1] = k4.y; kk[e4 + 2] = k4.z; kk[e4 + 3] = k4.w;
+                    qq[e4] = q4.x; qq[e4 + 1] = q4.y; qq[e4 + 2] = q4.z; qq[e4 + 3] = q4.w;
+                    ww[e4] = w4.x; ww[e4 + 1] = w4.y; ww[e4 + 2] = w4.z; ww[e4 + 3] = w4.w;
+                    uu[e4] = u4.x; uu[e4 + 1] = u4.y; uu[e4 + 2] = u4.z; uu[e4 + 3] = u4.w;
+                    bb[e4] = b4.x; bb[e4 + 1] = b4.y; bb[e4 + 2] = b4.z; bb[e4 + 3] = b4.w;
+                }
+                float r0 = 0.0f, r1 = 0.0f;
+#pragma unroll
+                for (int e = 0; e < DKQ; e += 2) { r0 = fmaf(S[e], uu[e], r0); r1 = fmaf(S[e + 1], uu[e + 1], r1); }
+                const float sa = LPC == 8 ? oct_sum(r0 + r1) : quad_sum(r0 + r1);
+                float o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+                for (int e = 0; e < DKQ; e += 2) {
+                    S[e] = fmaf(kk[e], vt, fmaf(ww[e], S[e], -bb[e] * sa)); o0 = fmaf(S[e], qq[e], o0);
+                    S[e + 1] = fmaf(kk[e + 1], vt, fmaf(ww[e + 1], S[e + 1], -bb[e + 1] * sa)); o1 = fmaf(S[e + 1], qq[e + 1], o1);
+                }
+                const float o = LPC == 8 ? oct_sum(o0 + o1) : quad_sum(o0 + o1);
+                if (live && rg == 0) P.out[(size_t)(sd.row0 + t0 + tt) * P.ldo + (size_t)h * P.dv + j] = o;
+            }
+        }
+        if (more) publish(buf ^ 1);
+        __syncthreads();
+    }
+    if (live) {
+#pragma unroll
+        for (int e = 0; e < DKQ; e++) state[(size_t)e * P.dv + j] = S[e];
+    }
+}
+
 // y[t][c] = o[t][c] / sqrt(mean_group(o^2) + eps) * w[c % wlen] * act(gate[t][c]); one workgroup per row, a wave per group
 __global__ void __launch_bounds__(256) k_gated_groupnorm(const float *__restrict__ o, size_t ldo, int C, int group, const bf16_t *__restrict__ w, int wlen,
                                                          const float *__restrict__ gate, size_t ldg, int gate_act, float eps, float *__restrict__ y,
@@ -522,6 +704,45 @@ int ifa_state_scan_f32(int kind, int in_act, const void *q_f32, size_t ldq, cons
         IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_state_scan<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(k_state_scan<1>, grid, dim3(64), smem, ifa_s(stream), P);
     }
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_chan_delta_gates_f32(const void *lr_f32, size_t ldl, int rank, const void *w2_bf16, const void *w0_bf16, float decay_mult, const void *a_f32, size_t lda,
+                             const void *k_f32, size_t ldk, int heads, int dim, float l2_eps, size_t rows, void *decay_f32, void *unit_f32, void *removal_f32,
+                             ifa_stream stream)
+{
+    IFA_REQUIRE(lr_f32 && w2_bf16 && a_f32 && k_f32 && decay_f32 && unit_f32 && removal_f32, "ifa_chan_delta_gates_f32: null pointer");
+    const size_t HD = (size_t)heads * dim;
+    IFA_REQUIRE(heads > 0 && dim > 0 && rows > 0 && rank >= 1 && rank <= 8192 && ldl >= (size_t)rank && lda >= HD && ldk >= HD, "ifa_chan_delta_gates_f32: bad shape");
+    hipLaunchKernelGGL(k_chan_delta_gates, dim3((unsigned)rows), dim3(256), (size_t)rank * 4, ifa_s(stream), (const float *)lr_f32, ldl, rank, (const bf16_t *)w2_bf16,
+                       (const bf16_t *)w0_bf16, decay_mult, (const float *)a_f32, lda, (const float *)k_f32, ldk, heads, dim, l2_eps, (float *)decay_f32, (float *)unit_f32,
+                       (float *)removal_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_state_scan_chan_f32(const void *q_f32, size_t ldq, const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int heads, int dk, int dv,
+                            const void *decay_f32, const void *unit_f32, const void *removal_f32, size_t ldg, const void *seqs_dev, int n_seqs,
+                            void *const *slot_base_dev, size_t state_off, void *out_f32, size_t ldo, ifa_stream stream)
+{
+    IFA_REQUIRE(q_f32 && k_f32 && v_f32 && decay_f32 && unit_f32 && removal_f32 && seqs_dev && slot_base_dev && out_f32, "ifa_state_scan_chan_f32: null pointer");
+    IFA_REQUIRE(heads > 0 && dk > 0 && dv > 0 && n_seqs > 0 && dk <= 64 * SCAN_DKL, "ifa_state_scan_chan_f32: bad shape (key size %d: at most %d)", dk, 64 * SCAN_DKL);
+    const size_t HK = (size_t)heads * dk, HV = (size_t)heads * dv;
+    IFA_REQUIRE(ldq >= HK && ldk >= HK && ldg >= HK && ldv >= HV && ldo >= HV, "ifa_state_scan_chan_f32: row strides too small");
+    ChanScanArgs P;
+    P.q = (const float *)q_f32; P.k = (const float *)k_f32; P.v = (const float *)v_f32; P.ldq = ldq; P.ldk = ldk; P.ldv = ldv;
+    P.w = (const float *)decay_f32; P.u = (const float *)unit_f32; P.b = (const float *)removal_f32; P.ldg = ldg;
+    P.heads = heads; P.dk = dk; P.dv = dv;
+    P.seqs = (const SeqDesc *)seqs_dev; P.slot_base = (float *const *)slot_base_dev; P.state_off = state_off;
+    P.out = (float *)out_f32; P.ldo = ldo;
+    const dim3 grid16((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 16)), grid8((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 8));
+#define IFA_CSCAN(DKV, L, G) if (dk == DKV) { hipLaunchKernelGGL((k_state_scan_chan_reg<DKV, L>), G, dim3(64), 0, ifa_s(stream), P); IFA_LAUNCH_CHECK(); return IFA_OK; }
+    IFA_CSCAN(16, 4, grid16) IFA_CSCAN(32, 4, grid16) IFA_CSCAN(48, 4, grid16) IFA_CSCAN(64, 8, grid8) IFA_CSCAN(96, 8, grid8) IFA_CSCAN(128, 8, grid8)
+#undef IFA_CSCAN
+    const size_t smem = ((size_t)dk * 64 + 5 * (size_t)dk) * 4;
+    IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_state_scan_chan, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(k_state_scan_chan, dim3((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 64)), dim3(64), smem, ifa_s(stream), P);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -23,6 +23,15 @@
 //                denominator; "kv_from": j = the layer has no key / value tensors and reads the cache rows of layer j
 // and a feed-forward of kind "dense" (clamped: min(gate, limit) * sigmoid(1.702 .) * (clamp(up) + 1)) or "moe" (router on logits + bias,
 // softmax over the chosen, gated SiLU experts, a shared expert times sigmoid(sg . h)), or none.
+//
+// Bogupel: width / vocab / norm.eps / embedding {scale, bigram {buckets, mul_prev, mul_cur}} / logit_scale / loop {start, stop, times}; the token
+// embedding times embedding.scale plus the hashed pair embedding; Dynamic Tanh norms (tanh(alpha x) w + b) in front of each sub-layer and of the
+// head; layers [loop.start, loop.stop) run loop.times times with the same weights, every pass on a cache of its own; mixer types
+//   "attention"      grouped queries, biases on q / k / v, weighted RMS norm of q and k per head, rotation of the first rot.dims dimensions with
+//                    frequencies scaled by wavelength (rot.scaling {factor, low, high, original}), values divided by their root mean square and
+//                    turned by their position over all of vdim (the head's output turned back), sliding window mask.size, a learned sink per head
+//   "general_delta"  generalized delta rule with a decay and a removal rate per head and key channel, per-head RMS norm, sigmoid gate
+// and a mixture of clamped gated experts (sigmoid scores, choice by score + correction, weights = the scores), or no feed-forward.
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -218,6 +227,121 @@ bool ParseSopulorn(const JsonValue &root, LayeredDesc &d)
     return true;
 }
 
+// ---- Bogupel
+bool ParseBogupel(const JsonValue &root, LayeredDesc &d)
+{
+    memset(&d.cfg, 0, sizeof(d.cfg));
+    if (!Need(root, "width", d.cfg.width, "config") || !Need(root, "vocab", d.cfg.vocab, "config")) return false;
+    const JsonValue *norm = root.Get("norm");
+    if (!norm || !Need(*norm, "eps", d.cfg.eps, "norm")) { if (!norm) EngineSetError("config.json: norm is missing"); return false; }
+    d.cfg.stem = 3;
+    d.cfg.embed_scale = 1.0f; d.cfg.logit_scale = 1.0f;
+    root.GetNumber("logit_scale", d.cfg.logit_scale);
+    if (const JsonValue *emb = root.Get("embedding")) {
+        emb->GetNumber("scale", d.cfg.embed_scale);
+        const JsonValue *bg = emb->Get("bigram");
+        if (bg && bg->type == JsonValue::Object
+            && (!Need(*bg, "buckets", d.cfg.bigram_buckets, "embedding.bigram") || !Need(*bg, "mul_prev", d.cfg.bigram_mul_prev, "embedding.bigram")
+                || !Need(*bg, "mul_cur", d.cfg.bigram_mul_cur, "embedding.bigram"))) return false;
+    }
+    const JsonValue *loop = root.Get("loop");
+    if (loop && loop->type == JsonValue::Object
+        && (!Need(*loop, "start", d.cfg.loop_start, "loop") || !Need(*loop, "stop", d.cfg.loop_stop, "loop") || !Need(*loop, "times", d.cfg.loop_times, "loop"))) return false;
+    const JsonValue *layers = root.Get("layers");
+    if (!layers || layers->type != JsonValue::Array || layers->arr.empty()) { EngineSetError("config.json: layers is missing or empty"); return false; }
+    for (size_t li = 0; li < layers->arr.size(); li++) {
+        const JsonValue &L = layers->arr[li];
+        ifa_layer_spec s; memset(&s, 0, sizeof(s));
+        std::string type;
+        const JsonValue *mx = L.Get("mixer");
+        if (!L.GetString("type", type) || !mx || mx->type != JsonValue::Object) { EngineSetError("config.json: layer %zu has no type / mixer", li); return false; }
+        s.block = IFA_BLOCK_PRENORM;
+        if (type == "attention") {
+            s.mixer = IFA_MIX_ROTARY;
+            s.a_sink = 2; s.a_vnorm = 1; s.a_vrot = 1;
+            if (!Need(*mx, "heads", s.a_heads, "mixer") || !Need(*mx, "kv_heads", s.a_kv_heads, "mixer") || !Need(*mx, "dim", s.a_dim, "mixer")
+                || !Need(*mx, "vdim", s.a_vdim, "mixer") || !Need(*mx, "scale", s.a_scale, "mixer")) return false;
+            const JsonValue *rot = mx->Get("rot");
+            if (!rot || rot->type != JsonValue::Object || !Need(*rot, "base", s.a_rot_base, "mixer.rot") || !Need(*rot, "dims", s.a_rot_dims, "mixer.rot")) {
+                if (!rot) EngineSetError("config.json: layer %zu: mixer.rot is missing", li);
+                return false;
+            }
+            const JsonValue *sc = rot->Get("scaling");
+            if (sc && sc->type == JsonValue::Object
+                && (!Need(*sc, "factor", s.a_rot_scale_factor, "rot.scaling") || !Need(*sc, "low", s.a_rot_scale_low, "rot.scaling")
+                    || !Need(*sc, "high", s.a_rot_scale_high, "rot.scaling") || !Need(*sc, "original", s.a_rot_scale_original, "rot.scaling"))) return false;
+            const JsonValue *mask = mx->Get("mask");
+            if (mask && mask->type == JsonValue::Object && !Need(*mask, "size", s.a_window, "mixer.mask")) return false;
+        } else if (type == "general_delta") {
+            s.mixer = IFA_MIX_CHAN_DELTA;
+            s.c_decay_mult = 0.60653065971263342f;      // exp(-1/2)
+            s.c_l2_eps = 1e-6f;
+            if (!Need(*mx, "heads", s.c_heads, "mixer") || !Need(*mx, "dim", s.c_dim, "mixer")) return false;
+        } else { EngineSetError("config.json: layer %zu: unknown type \"%s\"", li, type.c_str()); return false; }
+        const JsonValue *mlp = L.Get("mlp");
+        if (mlp && mlp->type == JsonValue::Object) {
+            std::string kind;
+            if (!mlp->GetString("kind", kind) || kind != "moe") { EngineSetError("config.json: layer %zu: mlp.kind \"%s\" is not supported (moe)", li, kind.c_str()); return false; }
+            const JsonValue *ex = mlp->Get("expert"), *ro = mlp->Get("router");
+            if (!ex || !ro) { EngineSetError("config.json: layer %zu: mlp needs expert and router", li); return false; }
+            s.ffn_kind = IFA_FFN_MOE; s.x_gated = 1; s.x_route = 0; s.x_score = 1; s.x_glu = 3;
+            if (!Need(*ex, "ff", s.x_ff, "mlp.expert") || !Need(*ex, "limit", s.x_limit, "mlp.expert") || !Need(*ro, "experts", s.x_experts, "mlp.router")
+                || !Need(*ro, "top", s.x_top, "mlp.router")) return false;
+        }
+        d.layers.push_back(s);
+        d.decays.push_back(std::vector<float>());
+    }
+    d.cfg.n_layers = (int)d.layers.size();
+    return true;
+}
+
+// the decay's bottleneck has the size its first matrix gives
+bool BogupelSizesFromTensors(const std::map<std::string, StTensorEntry> &index, LayeredDesc &d)
+{
+    for (size_t li = 0; li < d.layers.size(); li++) {
+        if (d.layers[li].mixer != IFA_MIX_CHAN_DELTA) continue;
+        const std::string name = "l" + std::to_string(li) + ".mix.w1";
+        auto it = index.find(name);
+        if (it == index.end() || it->second.shape.size() != 2 || it->second.shape[0] < 1) { EngineSetError("tensor %s is missing or not a matrix", name.c_str()); return false; }
+        d.layers[li].c_rank = (int)it->second.shape[0];
+    }
+    return true;
+}
+
+void BogupelNames(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out)
+{
+    out.push_back({"embed", {-1, IFA_T_EMBD}});
+    if (d.cfg.bigram_buckets > 0) out.push_back({"bigram", {-1, IFA_T_BIGRAM}});
+    if (d.cfg.loop_times > 0 && d.cfg.loop_start < d.cfg.loop_stop) out.push_back({"loop.step", {-1, IFA_T_LOOP_STEP}});
+    out.push_back({"final.norm", {-1, IFA_T_OUT_NORM}}); out.push_back({"final.norm.b", {-1, IFA_T_OUT_NORM_B}}); out.push_back({"final.norm.alpha", {-1, IFA_T_OUT_NORM_ALPHA}});
+    out.push_back({"head", {-1, IFA_T_LM_HEAD}});
+    for (size_t li = 0; li < d.layers.size(); li++) {
+        const ifa_layer_spec &s = d.layers[li];
+        const std::string p = "l" + std::to_string(li) + ".";
+        const int l = (int)li;
+        out.push_back({p + "norm1", {l, IFA_LT_NORM1}}); out.push_back({p + "norm1.b", {l, IFA_LT_NORM1_B}}); out.push_back({p + "norm1.alpha", {l, IFA_LT_NORM1_ALPHA}});
+        if (s.mixer == IFA_MIX_ROTARY) {
+            out.push_back({p + "mix.q", {l, IFA_LT_A_Q}}); out.push_back({p + "mix.q.b", {l, IFA_LT_A_Q_B}}); out.push_back({p + "mix.q.norm", {l, IFA_LT_A_Q_NORM}});
+            out.push_back({p + "mix.k", {l, IFA_LT_A_K}}); out.push_back({p + "mix.k.b", {l, IFA_LT_A_K_B}}); out.push_back({p + "mix.k.norm", {l, IFA_LT_A_K_NORM}});
+            out.push_back({p + "mix.v", {l, IFA_LT_A_V}}); out.push_back({p + "mix.v.b", {l, IFA_LT_A_V_B}});
+            out.push_back({p + "mix.sink", {l, IFA_LT_A_SINK}}); out.push_back({p + "mix.o", {l, IFA_LT_A_O}});
+        } else {
+            out.push_back({p + "mix.r", {l, IFA_LT_C_R}}); out.push_back({p + "mix.k", {l, IFA_LT_C_K}}); out.push_back({p + "mix.v", {l, IFA_LT_C_V}});
+            out.push_back({p + "mix.g", {l, IFA_LT_C_G}}); out.push_back({p + "mix.a", {l, IFA_LT_C_A}}); out.push_back({p + "mix.a.b", {l, IFA_LT_C_A_B}});
+            out.push_back({p + "mix.w1", {l, IFA_LT_C_W1}}); out.push_back({p + "mix.w2", {l, IFA_LT_C_W2}}); out.push_back({p + "mix.w0", {l, IFA_LT_C_W0}});
+            out.push_back({p + "mix.norm", {l, IFA_LT_C_NORM}}); out.push_back({p + "mix.o", {l, IFA_LT_C_O}});
+        }
+        if (!(s.ffn_kind == IFA_FFN_MOE && s.x_experts > 0)) continue;
+        out.push_back({p + "norm2", {l, IFA_LT_NORM2}}); out.push_back({p + "norm2.b", {l, IFA_LT_NORM2_B}}); out.push_back({p + "norm2.alpha", {l, IFA_LT_NORM2_ALPHA}});
+        out.push_back({p + "mlp.router", {l, IFA_LT_X_ROUTER}}); out.push_back({p + "mlp.correction", {l, IFA_LT_X_CORR}});
+        for (int e = 0; e < s.x_experts; e++) {      // per expert: its gate rows, then its up rows
+            out.push_back({p + "mlp.e" + std::to_string(e) + ".gate", {l, IFA_LT_X_UP}});
+            out.push_back({p + "mlp.e" + std::to_string(e) + ".up", {l, IFA_LT_X_UP}});
+        }
+        for (int e = 0; e < s.x_experts; e++) out.push_back({p + "mlp.e" + std::to_string(e) + ".down", {l, IFA_LT_X_DOWN}});
+    }
+}
+
 void SopulornNames(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out)
 {
     out.push_back({"embed", {-1, IFA_T_EMBD}});
@@ -337,7 +461,8 @@ struct ArchEntry {
 };
 const ArchEntry kArchitectures[] = {{"Gelarax", ParseGelarax, GelaraxSizesFromTensors, GelaraxNames},
                                     {"Muzopel", ParseMuzopel, NoSizesFromTensors, MuzopelNames},
-                                    {"Sopulorn", ParseSopulorn, NoSizesFromTensors, SopulornNames}};
+                                    {"Sopulorn", ParseSopulorn, NoSizesFromTensors, SopulornNames},
+                                    {"Bogupel", ParseBogupel, BogupelSizesFromTensors, BogupelNames}};
 
 const ArchEntry *FindArch(const std::string &name)
 {
