@@ -388,10 +388,18 @@ SOPULORN_SIZES = {  # --arch sopulorn: eight layers each (one with the dense fee
 }
 
 
+BOGUPEL_SIZES = {   # --arch bogupel: six layers in eight layer runs (attention, delta rule, a group of attention + delta rule that runs twice, attention, attention), a mixture of experts in every layer
+    "w1024": dict(width=1024, heads=8, kv_heads=2, dim=128, vdim=128, rot_dims=64, window=1024, delta_heads=8, delta_dim=128, rank=64, experts=16, top=4, ff=704),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, rot_dims=64, window=1024, delta_heads=16, delta_dim=128, rank=64, experts=32, top=6, ff=1408),
+}
+
+
 def run_arch_bench(args):
-    """--arch gelarax | muzopel | sopulorn: see run_gelarax_bench / run_muzopel_bench"""
+    """--arch gelarax | muzopel | sopulorn | bogupel: see run_gelarax_bench / run_muzopel_bench"""
     if args.arch.lower() == "muzopel":
         return run_muzopel_bench(args)
+    if args.arch.lower() == "bogupel":
+        return run_muzopel_bench(args, "bogupel")
     if args.arch.lower() == "sopulorn":
         return run_muzopel_bench(args, "sopulorn")
     return run_gelarax_bench(args)
@@ -421,17 +429,21 @@ def run_muzopel_bench(args, design="muzopel"):
         return time.perf_counter() - t0
 
     sop = design == "sopulorn"
-    label = "Sopulorn" if sop else "Muzopel"
+    label = design.capitalize()
+    size_table = {"sopulorn": SOPULORN_SIZES, "muzopel": MUZOPEL_SIZES, "bogupel": BOGUPEL_SIZES}[design]
+    make_cfg = {"sopulorn": synth.sopulorn_config, "muzopel": synth.muzopel_config, "bogupel": synth.bogupel_config}[design]
+    write_dir = {"sopulorn": synth.write_sopulorn_dir, "muzopel": synth.write_muzopel_dir, "bogupel": synth.write_bogupel_dir}[design]
+    shapes_of = {"sopulorn": synth.sopulorn_tensor_shapes, "muzopel": synth.muzopel_tensor_shapes, "bogupel": synth.bogupel_tensor_shapes}[design]
     for name in sizes:
-        sz = (SOPULORN_SIZES if sop else MUZOPEL_SIZES)[name]
-        cfg = synth.sopulorn_config(vocab=32000, **sz) if sop else synth.muzopel_config(vocab=32000, **sz)
+        sz = size_table[name]
+        cfg = make_cfg(vocab=32000, **sz)
         d = tempfile.mkdtemp(prefix="ifa_%s_" % design, dir="/dev/shm" if os.path.isdir("/dev/shm") else None)
         try:
-            (synth.write_sopulorn_dir if sop else synth.write_muzopel_dir)(d, cfg, seed=1)
+            write_dir(d, cfg, seed=1)
             eng = InferenceEngine.from_model_dir(d, "bfloat16", ctx, 2, False)
         finally:
             shutil.rmtree(d, ignore_errors=True)
-        shapes = synth.sopulorn_tensor_shapes(cfg) if sop else synth.muzopel_tensor_shapes(cfg)
+        shapes = shapes_of(cfg)
         g = {"prefill_tok_s": {}, "params": int(sum(int(np.prod(s)) for s in shapes.values()))}
         for n in lens:
             prompt = [int(t) for t in rng.integers(3, 32000, n)]
@@ -559,13 +571,13 @@ def main():
                     "a functional check of the N > 1 step logic on a one-GPU box, not a scaling number")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="CPU baseline sample size (0 = auto)")
-    ap.add_argument("--arch", default="", help="'gelarax', 'muzopel' or 'sopulorn': instead of the headline workload, prefill / decode rates of models of that design beside the "
+    ap.add_argument("--arch", default="", help="'gelarax', 'muzopel', 'sopulorn' or 'bogupel': instead of the headline workload, prefill / decode rates of models of that design beside the "
                     "closest standard model at equal size (one GPU; --prefill-lens, --steps, --warmup apply)")
     ap.add_argument("--arch-sizes", default="w1024,w2048")
     args = ap.parse_args()
     if args.arch:
-        if args.arch.lower() not in ("gelarax", "muzopel", "sopulorn"):
-            raise SystemExit("unknown --arch %s (gelarax, muzopel, sopulorn)" % args.arch)
+        if args.arch.lower() not in ("gelarax", "muzopel", "sopulorn", "bogupel"):
+            raise SystemExit("unknown --arch %s (gelarax, muzopel, sopulorn, bogupel)" % args.arch)
         if args.gpus > 1 or int(os.environ.get("WORLD_SIZE", "1")) > 1:
             raise SystemExit("--arch runs on one GPU")
         return run_arch_bench(args)

@@ -658,9 +658,9 @@ int ifa_moe_experts_gated_f32(const void *h_f32, size_t ldh, size_t rows, int wi
 /* Dynamic Tanh "norm": y[t][c] = tanh(alpha * x[t][c]) * w[c] + b[c]; alpha_bf16 one value, w / b bf16 [cols]; no mean, no variance */
 int ifa_dyt_f32(const void *x_f32, size_t ldx, size_t rows, size_t cols, const void *alpha_bf16, const void *w_bf16, const void *b_bf16, void *y_f32,
                 size_t ldy, ifa_stream stream);
-/* the residual update behind a sub-layer and the Dynamic Tanh in front of the next one in one launch: x += m (m null: skip), then
- * (w not null) h = tanh(alpha x) w + b */
-int ifa_add_dyt_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *alpha_bf16, const void *w_bf16,
+/* a residual update (behind a sub-layer, or at the start of a looped pass) and the Dynamic Tanh in front of the next sub-layer in one launch:
+ * x[t][c] += m[t][c] + vec[c] (either nullable), then (w not null) h = tanh(alpha x) w + b */
+int ifa_add_dyt_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *vec_bf16, const void *alpha_bf16, const void *w_bf16,
                     const void *b_bf16, void *h_f32, size_t ldh, ifa_stream stream);
 /* x[t][c] += (add_f32 ? add[t][c] : 0) + (vec_bf16 ? vec[c] : 0): what a pass of a looped layer group starts from */
 int ifa_add_rows_vec_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *add_f32, size_t lda, const void *vec_bf16, ifa_stream stream);
@@ -686,10 +686,14 @@ int ifa_attention_kv_sinks_f32(const void *q_f32, size_t ldq, int heads, int kv_
                                size_t ws_bytes, ifa_stream stream);
 /* gates of the generalized delta rule, per row and key channel c of heads * dim: decay[c] = exp(-decay_mult * sigmoid(w2[c] . tanh(lr) + w0[c]))
  * (lr fp32 [rows][rank]: the bottleneck's pre-activations; w2 bf16 [heads * dim][rank]; w0 bf16 [heads * dim], nullable), unit key
- * u = k / sqrt(sum_head(k^2) + l2_eps), removal[c] = sigmoid(a[c]) * u[c] (a with its bias already added).  Outputs fp32 [rows][heads * dim], contiguous. */
+ * u = k / sqrt(sum_head(k^2) + l2_eps), removal[c] = sigmoid(a[c]) * u[c] (a with its bias already added).  Outputs fp32 [rows][heads * dim], contiguous.
+ * rank 0: lr_f32 holds the sigmoid's argument itself, [rows][heads * dim] (w2 / w0 unused): larger steps form it as a matrix product over
+ * ifa_tanh_f32 of the bottleneck. */
 int ifa_chan_delta_gates_f32(const void *lr_f32, size_t ldl, int rank, const void *w2_bf16, const void *w0_bf16, float decay_mult, const void *a_f32, size_t lda,
                              const void *k_f32, size_t ldk, int heads, int dim, float l2_eps, size_t rows, void *decay_f32, void *unit_f32, void *removal_f32,
                              ifa_stream stream);
+/* x[t][c] = tanh(x[t][c]) in place, c < cols */
+int ifa_tanh_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, ifa_stream stream);
 /* generalized delta rule with a decay and a removal rate per key channel: per head, S [dk][dv] fp32 in the slot,
  * S <- diag(decay_t) S - removal_t (unit_t^T S) + k_t v_t^T (both terms read the old state), o_t = S^T q_t.
  * decay / unit / removal fp32 [rows][heads * dk] (row stride ldg).  dk <= 256. */
@@ -702,6 +706,10 @@ int ifa_moe_route_scores_f32(int score_kind, const void *logits_f32, size_t ld, 
                              void *wgt_f32, ifa_stream stream);
 int ifa_moe_route_rows_scores_f32(int score_kind, const void *h_f32, size_t ldh, size_t rows, int width, const void *router_bf16, int n_all, int top,
                                   const void *correction_bf16, int *idx_dev, void *wgt_f32, ifa_stream stream);
+/* the same with the Dynamic Tanh norm in front of the router inside the launch: h[t] = tanh(alpha x[t]) w + b is written (the experts read it), then routed */
+int ifa_moe_dyt_route_rows_f32(int score_kind, const void *x_f32, size_t ldx, const void *alpha_bf16, const void *norm_w_bf16, const void *norm_b_bf16, void *h_f32,
+                               size_t ldh, size_t rows, int width, const void *router_bf16, int n_all, int top, const void *correction_bf16, int *idx_dev,
+                               void *wgt_f32, ifa_stream stream);
 /* Gated experts with a choice of the gate: glu_kind 0 = silu(gate) * up (ifa_moe_experts_gated_f32), 3 = the clamped form of ifa_glu_ex_f32
  * (g = min(gate, limit), u = clamp(up, +-limit), g sigmoid(1.702 g) (u + 1)) */
 int ifa_moe_experts_glu_f32(int glu_kind, float limit, const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int top,

@@ -189,13 +189,15 @@ SIGNATURES = {
     "ifa_moe_route_top_f32": (_i, [_vp, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp]),
     "ifa_moe_experts_gated_f32": (_i, [_vp, _sz, _sz, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp, _sz, _i, _vp]),
     "ifa_dyt_f32": (_i, [_vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "ifa_add_dyt_f32": (_i, [_vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "ifa_add_dyt_f32": (_i, [_vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "ifa_moe_dyt_route_rows_f32": (_i, [_i, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _i, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "ifa_add_rows_vec_f32": (_i, [_vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp]),
     "ifa_embed_pair_scaled_f32": (_i, [_vp, _i, _i, _f, _vp, _i, _i, _i, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _vp]),
     "ifa_qkv_rope_store_f32": (_i, [_vp, _sz, _i, _vp, _sz, _vp, _sz, _i, _i, _i, _vp, _vp, _f, _i, _vp, _i, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _vp]),
     "ifa_rotate_heads_f32": (_i, [_vp, _sz, _i, _i, _i, _vp, _f, _vp, _vp, _sz, _vp]),
     "ifa_attention_kv_sinks_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _f, _i, _i, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _vp, _sz, _vp, _i, _i, _i, _vp, _sz, _vp]),
     "ifa_chan_delta_gates_f32": (_i, [_vp, _sz, _i, _vp, _vp, _f, _vp, _sz, _vp, _sz, _i, _i, _f, _sz, _vp, _vp, _vp, _vp]),
+    "ifa_tanh_f32": (_i, [_vp, _sz, _sz, _sz, _vp]),
     "ifa_state_scan_chan_f32": (_i, [_vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _vp, _vp, _vp, _sz, _vp, _i, _vp, _sz, _vp, _sz, _vp]),
     "ifa_moe_route_scores_f32": (_i, [_i, _vp, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp]),
     "ifa_moe_route_rows_scores_f32": (_i, [_i, _vp, _sz, _sz, _i, _vp, _i, _i, _vp, _vp, _vp, _vp]),

@@ -371,20 +371,23 @@ __global__ void __launch_bounds__(256) k_qk_rope_store(float *__restrict__ q, si
     const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
     const SeqDesc sd = seqs[row_seq[t]];
     const int pos = sd.pos0 + t - sd.row0, half = rot_dims / 2;
+    // VX: two workgroups per row, blockIdx.y 0 for the queries and keys, 1 for the values (each forms only the angles it needs)
+    const bool do_qk = !VX || blockIdx.y == 0, do_v = VX && blockIdx.y == 1;
+    if (do_qk)
     for (int i = tid; i < half; i += blockDim.x) {
         const double a = (double)pos * freq[i];
         cs[i] = (float)cos(a); cs[half + i] = (float)sin(a);
     }
     float *vcs = cs + 2 * half;
     const int vhalf = vdim / 2;
-    if (VX && k && v_freq) {
+    if (do_v && k && v_freq) {
         for (int i = tid; i < vhalf; i += blockDim.x) {
             const double a = (double)pos * v_freq[i];
             vcs[i] = (float)cos(a); vcs[vhalf + i] = (float)sin(a);
         }
     }
     __syncthreads();
-    const int n_items = heads + (k ? kv_heads : 0);
+    const int n_items = do_qk ? heads + (k ? kv_heads : 0) : 0;
     for (int it = wave; it < n_items; it += nw) {
         const bool is_q = it < heads;
         const int hd = is_q ? it : it - heads;
@@ -421,7 +424,7 @@ __global__ void __launch_bounds__(256) k_qk_rope_store(float *__restrict__ q, si
         }
     }
     if (VX) {
-        if (!k) return;
+        if (!k || !do_v) return;
         // a wave per value head: weightless RMS norm, then the turn by the position (a lane reads both members of a pair from the input row)
         for (int hd = wave; hd < kv_heads; hd += nw) {
             const float *src = v + (size_t)t * ldv + (size_t)hd * vdim;
@@ -596,7 +599,7 @@ int ifa_qkv_rope_store_f32(void *q_f32, size_t ldq, int heads, const void *k_f32
                 && (rot_dims == 0 || freq_f64_dev) && (!v_freq_f64_dev || vdim % 2 == 0), "ifa_qkv_rope_store_f32: bad shape (head sizes %d / %d, %d rotated)", dim, vdim, rot_dims);
     IFA_REQUIRE(ldq >= (size_t)heads * dim && (!k_f32 || (ldk >= (size_t)kv_heads * dim && ldv >= (size_t)kv_heads * vdim)), "ifa_qkv_rope_store_f32: row strides too small");
     const size_t smem = ((size_t)std::max(rot_dims, 2) + (size_t)vdim + 2) * 4;
-#define IFA_RS(N) hipLaunchKernelGGL((k_qk_rope_store<N, true>), dim3((unsigned)rows), dim3(256), smem, ifa_s(stream), (float *)q_f32, ldq, heads, \
+#define IFA_RS(N) hipLaunchKernelGGL((k_qk_rope_store<N, true>), dim3((unsigned)rows, k_f32 ? 2u : 1u), dim3(256), smem, ifa_s(stream), (float *)q_f32, ldq, heads, \
                                      (const float *)k_f32, ldk, (const float *)v_f32, ldv, kv_heads, dim, vdim, (const bf16_t *)q_norm_w_bf16, (const bf16_t *)k_norm_w_bf16, eps, \
                                      rot_dims, freq_f64_dev, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, k_off, v_off, v_norm ? 1 : 0, v_freq_f64_dev)
     if (dim <= 128) IFA_RS(2); else if (dim <= 256) IFA_RS(4); else IFA_RS(16);

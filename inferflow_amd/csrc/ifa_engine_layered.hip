@@ -479,7 +479,7 @@ int run_sandwich_layer(ifa_model *m, LLayer &L, size_t T, int nseq, bool h_ready
 
 // one PRENORM layer over T rows: x <- x + mixer(dyt1(x)); x <- x + experts(dyt2(x)), dyt(x) = tanh(alpha x) w + b.  pass: which copy of the
 // layer's cache rows / state (a layer of a looped group has one per pass).  The output products and the experts add into the residual themselves.
-int run_prenorm_layer(ifa_model *m, LLayer &L, size_t T, int nseq, int pass)
+int run_prenorm_layer(ifa_model *m, LLayer &L, size_t T, int nseq, int pass, bool pass_start)
 {
     LayeredNet *n = m->lay;
     const ifa_layered_config &c = n->cfg;
@@ -488,7 +488,11 @@ int run_prenorm_layer(ifa_model *m, LLayer &L, size_t T, int nseq, int pass)
     ifa_stream s = (ifa_stream)m->stream;
     void *const *slots = (void *const *)n->slot_base_dev;
     int rc;
-    if ((rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM1_ALPHA).data, L.T(IFA_LT_NORM1).data, L.T(IFA_LT_NORM1_B).data, n->h, W, s))) return rc;
+    // (the first layer of a looped pass: x += the embedding output, from the second pass on, + the pass's own vector, in the norm's launch)
+    if (pass_start) rc = ifa_add_dyt_f32(n->x, W, T, W, pass > 0 ? n->x0 : nullptr, W, (const bf16_t *)n->loop_step.data + (size_t)pass * W, L.T(IFA_LT_NORM1_ALPHA).data,
+                                         L.T(IFA_LT_NORM1).data, L.T(IFA_LT_NORM1_B).data, n->h, W, s);
+    else rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM1_ALPHA).data, L.T(IFA_LT_NORM1).data, L.T(IFA_LT_NORM1_B).data, n->h, W, s);
+    if (rc) return rc;
     if ((rc = linear(m, L.w_in, NI, W, n->h, W, T, L.b_in, nullptr, 1.0f, 0, n->proj, NI))) return rc;
     if (sp.mixer == IFA_MIX_ROTARY) {
         const int H = sp.a_heads, G = sp.a_kv_heads, D = sp.a_dim, DV = sp.a_vdim;
@@ -511,19 +515,28 @@ int run_prenorm_layer(ifa_model *m, LLayer &L, size_t T, int nseq, int pass)
     } else {
         const int H = sp.c_heads, D = sp.c_dim;
         const size_t CH = (size_t)H * D;
-        if ((rc = ifa_chan_delta_gates_f32(n->proj + L.c_cw, NI, sp.c_rank, L.T(IFA_LT_C_W2).data, L.T(IFA_LT_C_W0).data, sp.c_decay_mult, n->proj + L.c_ca, NI,
-                                           n->proj + L.c_ck, NI, H, D, sp.c_l2_eps, T, n->cg_decay, n->cg_unit, n->cg_rem, s))) return rc;
+        if (T <= 8) {      // a few rows: the bottleneck's second matrix inside the gates' launch
+            if ((rc = ifa_chan_delta_gates_f32(n->proj + L.c_cw, NI, sp.c_rank, L.T(IFA_LT_C_W2).data, L.T(IFA_LT_C_W0).data, sp.c_decay_mult, n->proj + L.c_ca, NI,
+                                               n->proj + L.c_ck, NI, H, D, sp.c_l2_eps, T, n->cg_decay, n->cg_unit, n->cg_rem, s))) return rc;
+        } else {           // the sigmoid's argument as a product on the matrix cores (its bias = w0), left where the decays will be written
+            if ((rc = ifa_tanh_f32(n->proj + L.c_cw, NI, T, (size_t)sp.c_rank, s))) return rc;
+            // (fp32 operands in both modes: the product is small, and a decay close to one carries an error of its argument through hundreds of tokens)
+            if ((rc = ifa_linear_bf16w(L.T(IFA_LT_C_W2).data, CH, (size_t)sp.c_rank, n->proj + L.c_cw, NI, T, L.T(IFA_LT_C_W0).data, nullptr, 1.0f, 0, 1, n->cg_decay, CH, 0, 0, s))) return rc;
+            if ((rc = ifa_chan_delta_gates_f32(n->cg_decay, CH, 0, nullptr, nullptr, sp.c_decay_mult, n->proj + L.c_ca, NI, n->proj + L.c_ck, NI, H, D, sp.c_l2_eps, T,
+                                               n->cg_decay, n->cg_unit, n->cg_rem, s))) return rc;
+        }
         if ((rc = ifa_state_scan_chan_f32(n->proj + L.c_cr, NI, n->proj + L.c_ck, NI, n->proj + L.c_cv, NI, H, D, D, n->cg_decay, n->cg_unit, n->cg_rem, CH, n->seqs_dev, nseq,
                                           slots, L.o_rec + po, n->m1, CH, s))) return rc;
         if ((rc = ifa_gated_groupnorm_f32(n->m1, CH, T, (int)CH, D, L.T(IFA_LT_C_NORM).data, (int)CH, n->proj + L.c_cg, NI, 0, c.eps, n->m1, CH, s))) return rc;
         if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_C_O).data, W, CH, n->m1, CH, T, nullptr, nullptr, 1.0f, 1, n->x, W))) return rc;
     }
     if (!has_moe(sp)) return IFA_OK;
-    if ((rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM2_ALPHA).data, L.T(IFA_LT_NORM2).data, L.T(IFA_LT_NORM2_B).data, n->h, W, s))) return rc;
     const int XA = sp.x_experts;
-    if (T <= 8 && XA <= 512) {      // a few rows: the router's product inside the choice's launch
-        if ((rc = ifa_moe_route_rows_scores_f32(sp.x_score, n->h, W, T, (int)W, L.T(IFA_LT_X_ROUTER).data, XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
+    if (T <= 8 && XA <= 512) {      // a few rows: the norm and the router's product inside the choice's launch
+        if ((rc = ifa_moe_dyt_route_rows_f32(sp.x_score, n->x, W, L.T(IFA_LT_NORM2_ALPHA).data, L.T(IFA_LT_NORM2).data, L.T(IFA_LT_NORM2_B).data, n->h, W, T, (int)W,
+                                             L.T(IFA_LT_X_ROUTER).data, XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
     } else {
+        if ((rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM2_ALPHA).data, L.T(IFA_LT_NORM2).data, L.T(IFA_LT_NORM2_B).data, n->h, W, s))) return rc;
         if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_X_ROUTER).data, (size_t)XA, W, n->h, W, T, nullptr, nullptr, 1.0f, 0, n->m2, (size_t)XA))) return rc;
         if ((rc = ifa_moe_route_scores_f32(sp.x_score, n->m2, (size_t)XA, T, XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
     }
@@ -560,10 +573,9 @@ int run_layers(ifa_model *m, size_t T, int nseq)
         const ifa_layer_spec &sp = L.spec;
         const LLayer *next_layer = ri + 1 < n->runs.size() ? &n->layers[(size_t)n->runs[ri + 1].first] : nullptr;
         // a pass of the looped group starts from x (+ the embedding output, from the second pass on) + the pass's own vector
-        if (c.loop_times > 0 && (int)li == c.loop_start && c.loop_start < c.loop_stop
-            && (rc = ifa_add_rows_vec_f32(n->x, W, T, W, pass > 0 ? n->x0 : nullptr, W, (const bf16_t *)n->loop_step.data + (size_t)pass * W, s))) return rc;
+        const bool pass_start = c.loop_times > 0 && (int)li == c.loop_start && c.loop_start < c.loop_stop;
         if (sp.block == IFA_BLOCK_PRENORM) {
-            if ((rc = run_prenorm_layer(m, L, T, nseq, pass))) return rc;
+            if ((rc = run_prenorm_layer(m, L, T, nseq, pass, pass_start))) return rc;
             h_ready = false;
             if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
                 IFA_HIP_CHECK(hipMemcpyAsync(n->taps + ri * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));

@@ -84,13 +84,21 @@ __global__ void __launch_bounds__(64) k_moe_route_top(const float *__restrict__ 
 
 // Steps of a few rows: the router's product and its choice in one launch.  A workgroup per row: the waves share out the router's outputs
 // (a dot of `width` each), then the scores and the `top` passes as in k_moe_route (wave 0; the other waves only keep the barriers).
-__global__ void __launch_bounds__(1024) k_moe_route_rows(const float *__restrict__ h, size_t ldh, int W, const bf16_t *__restrict__ router, int n_all, int top,
-                                                        const bf16_t *__restrict__ corr, int *__restrict__ idx, float *__restrict__ wgt, int vec, int score_kind)
+// (x not null: the row the router reads is formed here first, h[t] = tanh(alpha x[t]) nw + nb, and written for the experts behind)
+__global__ void __launch_bounds__(1024) k_moe_route_rows(const float *h, size_t ldh, int W, const bf16_t *__restrict__ router, int n_all, int top,
+                                                        const bf16_t *__restrict__ corr, int *__restrict__ idx, float *__restrict__ wgt, int vec, int score_kind,
+                                                        const float *__restrict__ x, size_t ldx, const bf16_t *__restrict__ alpha, const bf16_t *__restrict__ nw_,
+                                                        const bf16_t *__restrict__ nb_, float *h_out)
 {
     extern __shared__ float sc[];          // [n_all] logits, then scores; [n_all] choice scores
     float *ch = sc + n_all;
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const float *hr = h + (size_t)t * ldh;
+    if (x) {
+        const float a = bf2f(alpha[0]);
+        for (int c = threadIdx.x; c < W; c += blockDim.x) h_out[(size_t)t * ldh + c] = fmaf(tanhf(a * x[(size_t)t * ldx + c]), bf2f(nw_[c]), bf2f(nb_[c]));
+        __syncthreads();          // (the workgroup reads back what it has written itself)
+    }
     for (int e = wave; e < n_all; e += nw) {
         const bf16_t *w = router + (size_t)e * W;
         float acc = 0.0f;
@@ -336,7 +344,23 @@ int ifa_moe_route_rows_scores_f32(int score_kind, const void *h_f32, size_t ldh,
                 "ifa_moe_route_rows_f32: bad shape");
     const int vec = (width % 8 == 0 && ldh % 4 == 0 && ((uintptr_t)h_f32 & 15) == 0 && ((uintptr_t)router_bf16 & 15) == 0) ? 1 : 0;
     hipLaunchKernelGGL(k_moe_route_rows, dim3((unsigned)rows), dim3(n_all > 8 ? 1024 : 256), (size_t)n_all * 8, ifa_s(stream), (const float *)h_f32, ldh, width,
-                       (const bf16_t *)router_bf16, n_all, top, (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32, vec, score_kind);
+                       (const bf16_t *)router_bf16, n_all, top, (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32, vec, score_kind, (const float *)nullptr, (size_t)0,
+                       (const bf16_t *)nullptr, (const bf16_t *)nullptr, (const bf16_t *)nullptr, (float *)nullptr);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_moe_dyt_route_rows_f32(int score_kind, const void *x_f32, size_t ldx, const void *alpha_bf16, const void *norm_w_bf16, const void *norm_b_bf16, void *h_f32,
+                               size_t ldh, size_t rows, int width, const void *router_bf16, int n_all, int top, const void *correction_bf16, int *idx_dev,
+                               void *wgt_f32, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && alpha_bf16 && norm_w_bf16 && norm_b_bf16 && h_f32 && router_bf16 && idx_dev && wgt_f32 && x_f32 != h_f32, "ifa_moe_dyt_route_rows_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && rows <= 64 && width > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ldh >= (size_t)width && ldx >= (size_t)width
+                && (score_kind == 0 || score_kind == 1), "ifa_moe_dyt_route_rows_f32: bad shape");
+    const int vec = (width % 8 == 0 && ldh % 4 == 0 && ((uintptr_t)h_f32 & 15) == 0 && ((uintptr_t)router_bf16 & 15) == 0) ? 1 : 0;
+    hipLaunchKernelGGL(k_moe_route_rows, dim3((unsigned)rows), dim3(n_all > 8 ? 1024 : 256), (size_t)n_all * 8, ifa_s(stream), (const float *)h_f32, ldh, width,
+                       (const bf16_t *)router_bf16, n_all, top, (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32, vec, score_kind, (const float *)x_f32, ldx,
+                       (const bf16_t *)alpha_bf16, (const bf16_t *)norm_w_bf16, (const bf16_t *)norm_b_bf16, (float *)h_f32);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -117,15 +117,19 @@ __global__ void __launch_bounds__(256) k_dyt(const float *__restrict__ x, size_t
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < cols; c += gridDim.y * blockDim.x) yr[c] = fmaf(tanhf(a * xr[c]), bf2f(w[c]), bf2f(b[c]));
 }
 
-// x += m, then h = tanh(alpha x) w + b: the residual update behind a sub-layer and the norm in front of the next one
-__global__ void __launch_bounds__(256) k_add_dyt(float *__restrict__ x, size_t ldx, int cols, const float *__restrict__ m, size_t ldm, const bf16_t *__restrict__ alpha,
-                                                 const bf16_t *__restrict__ w, const bf16_t *__restrict__ b, float *__restrict__ h, size_t ldh)
+// x += m + vec, then h = tanh(alpha x) w + b: the residual update behind a sub-layer (or the start of a looped pass) and the norm in front of the next one
+__global__ void __launch_bounds__(256) k_add_dyt(float *__restrict__ x, size_t ldx, int cols, const float *__restrict__ m, size_t ldm, const bf16_t *__restrict__ vec,
+                                                 const bf16_t *__restrict__ alpha, const bf16_t *__restrict__ w, const bf16_t *__restrict__ b, float *__restrict__ h, size_t ldh)
 {
     const float a = w ? bf2f(alpha[0]) : 0.0f;
     float *xr = x + (size_t)blockIdx.x * ldx;
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < cols; c += gridDim.y * blockDim.x) {
         float v = xr[c];
-        if (m) { v += m[(size_t)blockIdx.x * ldm + c]; xr[c] = v; }
+        if (m || vec) {
+            if (m) v += m[(size_t)blockIdx.x * ldm + c];
+            if (vec) v += bf2f(vec[c]);
+            xr[c] = v;
+        }
         if (w) h[(size_t)blockIdx.x * ldh + c] = fmaf(tanhf(a * v), bf2f(w[c]), bf2f(b[c]));
     }
 }
@@ -378,13 +382,13 @@ int ifa_dyt_f32(const void *x_f32, size_t ldx, size_t rows, size_t cols, const v
     return IFA_OK;
 }
 
-int ifa_add_dyt_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *alpha_bf16, const void *w_bf16,
+int ifa_add_dyt_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *vec_bf16, const void *alpha_bf16, const void *w_bf16,
                     const void *b_bf16, void *h_f32, size_t ldh, ifa_stream stream)
 {
     IFA_REQUIRE(x_f32 && (!w_bf16 || (alpha_bf16 && b_bf16 && h_f32)), "ifa_add_dyt_f32: null pointer");
     IFA_REQUIRE(rows > 0 && rows < (1u << 31) && cols > 0 && ldx >= cols && (!m_f32 || ldm >= cols) && (!w_bf16 || ldh >= cols), "ifa_add_dyt_f32: bad arguments");
-    if (!m_f32 && !w_bf16) return IFA_OK;
-    hipLaunchKernelGGL(k_add_dyt, rows_grid(rows, cols), dim3(256), 0, ifa_s(stream), (float *)x_f32, ldx, (int)cols, (const float *)m_f32, ldm,
+    if (!m_f32 && !vec_bf16 && !w_bf16) return IFA_OK;
+    hipLaunchKernelGGL(k_add_dyt, rows_grid(rows, cols), dim3(256), 0, ifa_s(stream), (float *)x_f32, ldx, (int)cols, (const float *)m_f32, ldm, (const bf16_t *)vec_bf16,
                        (const bf16_t *)alpha_bf16, (const bf16_t *)w_bf16, (const bf16_t *)b_bf16, (float *)h_f32, ldh);
     IFA_LAUNCH_CHECK();
     return IFA_OK;

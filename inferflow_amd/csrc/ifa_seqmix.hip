@@ -374,35 +374,54 @@ __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
 // ---- generalized delta rule with a decay and a removal rate per key channel:
 //   S <- diag(w_t) S - b_t (u_t^T S) + k_t v_t^T   (both terms read the old state),   o_t = S^T q_t
 // w (decay), u (unit key) and b (removal rate times unit key) come per row and key channel from k_chan_delta_gates.
-// one workgroup per row: the bottleneck's activations tanh(lr) in LDS, then a wave per head at a time:
-// decay = exp(-mult * sigmoid(w2[c] . tanh(lr) + w0[c])), u = k / sqrt(sum k^2 + l2_eps), b = sigmoid(a) * u
-__global__ void __launch_bounds__(256) k_chan_delta_gates(const float *__restrict__ lr, size_t ldl, int rank, const bf16_t *__restrict__ w2, const bf16_t *__restrict__ w0,
+// grid (rows, heads): a workgroup per head of a row.  The bottleneck's activations tanh(lr) in LDS, then a thread per key channel:
+// decay = exp(-mult * sigmoid(w2[c] . tanh(lr) + w0[c])), u = k / sqrt(sum k^2 + l2_eps), b = sigmoid(a) * u.
+// rank 0: lr holds the sigmoid's argument itself, [heads * dim] per row (larger steps form it as a matrix product).
+__global__ void __launch_bounds__(256) k_chan_delta_gates(const float *lr, size_t ldl, int rank, const bf16_t *__restrict__ w2, const bf16_t *__restrict__ w0,
                                                           float mult, const float *__restrict__ a, size_t lda, const float *__restrict__ k, size_t ldk, int H, int D,
-                                                          float l2_eps, float *__restrict__ decay, float *__restrict__ unit, float *__restrict__ removal)
+                                                          float l2_eps, float *decay, float *__restrict__ unit, float *__restrict__ removal, int vec)      // (rank 0: decay may be lr itself)
 {
     extern __shared__ float th[];          // [rank]
-    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __shared__ float red[17];
+    const int t = blockIdx.x, h = blockIdx.y;
     for (int i = threadIdx.x; i < rank; i += blockDim.x) th[i] = tanhf(lr[(size_t)t * ldl + i]);
-    __syncthreads();
     const size_t HD = (size_t)H * D;
-    for (int h = wave; h < H; h += nw) {
-        const float *kr = k + (size_t)t * ldk + (size_t)h * D;
-        float s = 0.0f;
-        for (int c = lane; c < D; c += 64) s = fmaf(kr[c], kr[c], s);
-        const float rinv = 1.0f / sqrtf(wave_sum(s) + l2_eps);
-        for (int c = lane; c < D; c += 64) {
-            const size_t hc = (size_t)h * D + c;
+    const float *kr = k + (size_t)t * ldk + (size_t)h * D;
+    float s = 0.0f;
+    for (int c = threadIdx.x; c < D; c += blockDim.x) s = fmaf(kr[c], kr[c], s);
+    const float rinv = 1.0f / sqrtf(block_sum(s, red) + l2_eps);          // (its barriers also publish th)
+    for (int c = threadIdx.x; c < D; c += blockDim.x) {
+        const size_t hc = (size_t)h * D + c;
+        float z;
+        if (rank > 0) {
             const bf16_t *wr = w2 + hc * (size_t)rank;
             float z0 = w0 ? bf2f(w0[hc]) : 0.0f, z1 = 0.0f;
             int i = 0;
+            if (vec) {          // rows of whole 16-byte pieces
+                for (; i + 8 <= rank; i += 8) {
+                    const uint4 wv = *reinterpret_cast<const uint4 *>(wr + i);
+                    z0 = fmaf(__uint_as_float(wv.x << 16), th[i], z0); z1 = fmaf(__uint_as_float(wv.x & 0xFFFF0000u), th[i + 1], z1);
+                    z0 = fmaf(__uint_as_float(wv.y << 16), th[i + 2], z0); z1 = fmaf(__uint_as_float(wv.y & 0xFFFF0000u), th[i + 3], z1);
+                    z0 = fmaf(__uint_as_float(wv.z << 16), th[i + 4], z0); z1 = fmaf(__uint_as_float(wv.z & 0xFFFF0000u), th[i + 5], z1);
+                    z0 = fmaf(__uint_as_float(wv.w << 16), th[i + 6], z0); z1 = fmaf(__uint_as_float(wv.w & 0xFFFF0000u), th[i + 7], z1);
+                }
+            }
             for (; i + 1 < rank; i += 2) { z0 = fmaf(bf2f(wr[i]), th[i], z0); z1 = fmaf(bf2f(wr[i + 1]), th[i + 1], z1); }
             if (i < rank) z0 = fmaf(bf2f(wr[i]), th[i], z0);
-            const float u = kr[c] * rinv;
-            decay[(size_t)t * HD + hc] = expf(-mult * sigmoid_f(z0 + z1));
-            unit[(size_t)t * HD + hc] = u;
-            removal[(size_t)t * HD + hc] = sigmoid_f(a[(size_t)t * lda + hc]) * u;
-        }
+            z = z0 + z1;
+        } else z = lr[(size_t)t * ldl + hc];
+        const float u = kr[c] * rinv;
+        decay[(size_t)t * HD + hc] = expf(-mult * sigmoid_f(z));
+        unit[(size_t)t * HD + hc] = u;
+        removal[(size_t)t * HD + hc] = sigmoid_f(a[(size_t)t * lda + hc]) * u;
     }
+}
+
+// x[t][c] = tanh(x[t][c]) in place over a column range of the rows
+__global__ void __launch_bounds__(256) k_tanh_cols(float *__restrict__ x, size_t ldx, int cols)
+{
+    float *xr = x + (size_t)blockIdx.x * ldx;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) xr[c] = tanhf(xr[c]);
 }
 
 struct ChanScanArgs {
@@ -712,12 +731,23 @@ int ifa_chan_delta_gates_f32(const void *lr_f32, size_t ldl, int rank, const voi
                              const void *k_f32, size_t ldk, int heads, int dim, float l2_eps, size_t rows, void *decay_f32, void *unit_f32, void *removal_f32,
                              ifa_stream stream)
 {
-    IFA_REQUIRE(lr_f32 && w2_bf16 && a_f32 && k_f32 && decay_f32 && unit_f32 && removal_f32, "ifa_chan_delta_gates_f32: null pointer");
+    IFA_REQUIRE(lr_f32 && (rank == 0 || w2_bf16) && a_f32 && k_f32 && decay_f32 && unit_f32 && removal_f32, "ifa_chan_delta_gates_f32: null pointer");
     const size_t HD = (size_t)heads * dim;
-    IFA_REQUIRE(heads > 0 && dim > 0 && rows > 0 && rank >= 1 && rank <= 8192 && ldl >= (size_t)rank && lda >= HD && ldk >= HD, "ifa_chan_delta_gates_f32: bad shape");
-    hipLaunchKernelGGL(k_chan_delta_gates, dim3((unsigned)rows), dim3(256), (size_t)rank * 4, ifa_s(stream), (const float *)lr_f32, ldl, rank, (const bf16_t *)w2_bf16,
-                       (const bf16_t *)w0_bf16, decay_mult, (const float *)a_f32, lda, (const float *)k_f32, ldk, heads, dim, l2_eps, (float *)decay_f32, (float *)unit_f32,
-                       (float *)removal_f32);
+    IFA_REQUIRE(heads > 0 && dim > 0 && rows > 0 && rank >= 0 && rank <= 8192 && ldl >= (rank > 0 ? (size_t)rank : HD) && lda >= HD && ldk >= HD,
+                "ifa_chan_delta_gates_f32: bad shape");
+    IFA_REQUIRE(heads < 65536, "ifa_chan_delta_gates_f32: %d heads", heads);
+    const int vec = (rank % 8 == 0 && ((uintptr_t)w2_bf16 & 15) == 0) ? 1 : 0;
+    hipLaunchKernelGGL(k_chan_delta_gates, dim3((unsigned)rows, (unsigned)heads), dim3(dim <= 64 ? 64 : (dim <= 128 ? 128 : 256)), (size_t)rank * 4, ifa_s(stream),
+                       (const float *)lr_f32, ldl, rank, (const bf16_t *)w2_bf16, (const bf16_t *)w0_bf16, decay_mult, (const float *)a_f32, lda, (const float *)k_f32, ldk,
+                       heads, dim, l2_eps, (float *)decay_f32, (float *)unit_f32, (float *)removal_f32, vec);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_tanh_f32(void *x_f32, size_t ldx, size_t rows, size_t cols, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && rows > 0 && rows < (1u << 31) && cols > 0 && ldx >= cols, "ifa_tanh_f32: bad arguments");
+    hipLaunchKernelGGL(k_tanh_cols, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (float *)x_f32, ldx, (int)cols);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -254,6 +254,54 @@ def sopulorn_tensor_shapes(cfg):
     return s
 
 
+def bogupel_config(width=2048, vocab=32000, heads=16, kv_heads=4, dim=128, vdim=128, rot_dims=64, window=1024, delta_heads=16, delta_dim=128, rank=64, experts=32, top=6,
+                   ff=1408):
+    """six layers, eight layer runs: attention, delta rule, a looped group of (attention, delta rule) that runs twice, attention, attention; a mixture of clamped
+    gated experts in every layer"""
+    moe = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}
+    att = {"type": "attention", "mlp": moe,
+           "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": float(dim ** -0.5), "mask": {"size": window},
+                     "rot": {"base": 10000.0, "dims": rot_dims, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+    dlt = {"type": "general_delta", "mlp": moe, "mixer": {"heads": delta_heads, "dim": delta_dim}, "_rank": rank}
+    return {"architecture": "Bogupel", "width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "logit_scale": 0.5, "loop": {"start": 2, "stop": 4, "times": 2},
+            "embedding": {"scale": 4.0, "bigram": {"buckets": 65521, "mul_prev": 31337, "mul_cur": 7919}}, "layers": [att, dlt, att, dlt, att, att]}
+
+
+def bogupel_tensor_shapes(cfg):
+    W_, V = cfg["width"], cfg["vocab"]
+    s = {"embed": (V, W_), "final.norm": (W_,), "final.norm.b": (W_,), "final.norm.alpha": (), "head": (V, W_)}
+    bg = (cfg.get("embedding") or {}).get("bigram")
+    if bg:
+        s["bigram"] = (bg["buckets"] + 1, W_)
+    if cfg.get("loop"):
+        s["loop.step"] = (cfg["loop"]["times"], W_)
+    for li, L in enumerate(cfg["layers"]):
+        p, m = "l%d." % li, L["mixer"]
+        s.update({p + "norm1": (W_,), p + "norm1.b": (W_,), p + "norm1.alpha": ()})
+        if L["type"] == "attention":
+            H, G, D, DV = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            s.update({p + "mix.q": (H * D, W_), p + "mix.q.b": (H * D,), p + "mix.q.norm": (D,), p + "mix.k": (G * D, W_), p + "mix.k.b": (G * D,), p + "mix.k.norm": (D,),
+                      p + "mix.v": (G * DV, W_), p + "mix.v.b": (G * DV,), p + "mix.sink": (H,), p + "mix.o": (W_, H * DV)})
+        else:
+            C, R = m["heads"] * m["dim"], L.get("_rank", 64)
+            s.update({p + "mix.r": (C, W_), p + "mix.k": (C, W_), p + "mix.v": (C, W_), p + "mix.g": (C, W_), p + "mix.a": (C, W_), p + "mix.a.b": (C,), p + "mix.w1": (R, W_),
+                      p + "mix.w2": (C, R), p + "mix.w0": (C,), p + "mix.norm": (C,), p + "mix.o": (W_, C)})
+        mlp = L.get("mlp")
+        if not mlp:
+            continue
+        E, F = mlp["router"]["experts"], mlp["expert"]["ff"]
+        s.update({p + "norm2": (W_,), p + "norm2.b": (W_,), p + "norm2.alpha": (), p + "mlp.router": (E, W_), p + "mlp.correction": (E,)})
+        for e in range(E):
+            s.update({p + "mlp.e%d.gate" % e: (F, W_), p + "mlp.e%d.up" % e: (F, W_), p + "mlp.e%d.down" % e: (W_, F)})
+    return s
+
+
+def write_bogupel_dir(path, cfg, seed=0):
+    clean = dict(cfg)
+    clean["layers"] = [{k: v for k, v in L.items() if not k.startswith("_")} for L in cfg["layers"]]
+    return write_gelarax_dir(path, clean, seed, bogupel_tensor_shapes(cfg))
+
+
 def write_sopulorn_dir(path, cfg, seed=0):
     return write_gelarax_dir(path, cfg, seed, sopulorn_tensor_shapes(cfg))
 
@@ -289,6 +337,8 @@ def write_gelarax_dir(path, cfg, seed=0, shapes=None):
                 a = 0.05 * rng.standard_normal(shape, dtype=np.float32)          # (this design's norms multiply by one plus the stored weight)
             elif len(shape) == 1 and leaf in ("norm1", "norm2", "norm", "ls1", "ls2"):
                 a = 1.0 + 0.05 * rng.standard_normal(shape, dtype=np.float32)
+            elif leaf == "alpha":
+                a = np.full(shape, 0.5, np.float32)          # (the scalar of an element-wise tanh norm)
             elif leaf == "dwa":
                 a = np.full(shape, 1.0 / shape[0], np.float32)
             elif leaf == "correction":

@@ -43,7 +43,7 @@ def test_dynamic_tanh_store_after_an_update_and_the_start_of_a_pass(rows, cols):
     assert np.abs(got[:, :cols] - want).max() < 2e-6 * max(1.0, np.abs(want).max()) and np.all(got[:, cols:] == 7.0)
     # x += m; h = dyt(x)
     xd, h = dev32(x), torch.full((rows, cols), 7.0, dtype=torch.float32, device="cuda")
-    ia.check(L.ifa_add_dyt_f32(p(xd), cols + 3, rows, cols, p(dev32(m)), cols + 2, p(devbf(alpha)), p(devbf(w)), p(devbf(b)), p(h), cols, None)); sync()
+    ia.check(L.ifa_add_dyt_f32(p(xd), cols + 3, rows, cols, p(dev32(m)), cols + 2, None, p(devbf(alpha)), p(devbf(w)), p(devbf(b)), p(h), cols, None)); sync()
     xs = x[:, :cols] + m[:, :cols]
     assert np.array_equal(xd.cpu().numpy()[:, :cols], xs) and np.array_equal(xd.cpu().numpy()[:, cols:], x[:, cols:])
     want2 = orc.dyt(orc.f64(xs), alpha, orc.f64(w), orc.f64(b))
