@@ -55,6 +55,14 @@ __device__ __forceinline__ float oct_sum(float v)
     return v;
 }
 
+// sum over the sixteen lanes 16 q .. 16 q + 15 (a DPP row): the oct sums, then the other half's through a rotation of the row by 8
+__device__ __forceinline__ float hex_sum(float v)
+{
+    v = oct_sum(v);
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x128, 0xF, 0xF, true));
+    return v;
+}
+
 // sum over a workgroup of up to 1024 threads; red: 17 floats of LDS; every thread gets the result
 __device__ __forceinline__ float block_sum(float v, float *red)
 {

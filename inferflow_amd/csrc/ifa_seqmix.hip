@@ -480,7 +480,8 @@ __global__ void __launch_bounds__(64) k_state_scan_chan(ChanScanArgs P)
     if (live) for (int i = 0; i < dk; i++) state[(size_t)i * P.dv + j] = S[i * 64 + lane];
 }
 
-// key sizes 16 / 32 / 48 / 64 / 96 / 128: the state in registers, LPC lanes per column (as k_state_scan_reg), token groups of SCAN_TB staged in LDS
+// key sizes 16 / 32 / 48 / 64 / 96 / 128: the state in registers, LPC lanes per column (as k_state_scan_reg; sixteen lanes from 128 key channels on, so
+// that a lane walks eight rows of its column per token and a head's columns are spread over twice as many waves), token groups of SCAN_TB staged in LDS
 template <int DK, int LPC>
 __global__ void __launch_bounds__(64) k_state_scan_chan_reg(ChanScanArgs P)
 {
@@ -550,14 +551,14 @@ __global__ void __launch_bounds__(64) k_state_scan_chan_reg(ChanScanArgs P)
                 float r0 = 0.0f, r1 = 0.0f;
 #pragma unroll
                 for (int e = 0; e < DKQ; e += 2) { r0 = fmaf(S[e], uu[e], r0); r1 = fmaf(S[e + 1], uu[e + 1], r1); }
-                const float sa = LPC == 8 ? oct_sum(r0 + r1) : quad_sum(r0 + r1);
+                const float sa = LPC == 16 ? hex_sum(r0 + r1) : (LPC == 8 ? oct_sum(r0 + r1) : quad_sum(r0 + r1));
                 float o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
                 for (int e = 0; e < DKQ; e += 2) {
                     S[e] = fmaf(kk[e], vt, fmaf(ww[e], S[e], -bb[e] * sa)); o0 = fmaf(S[e], qq[e], o0);
                     S[e + 1] = fmaf(kk[e + 1], vt, fmaf(ww[e + 1], S[e + 1], -bb[e + 1] * sa)); o1 = fmaf(S[e + 1], qq[e + 1], o1);
                 }
-                const float o = LPC == 8 ? oct_sum(o0 + o1) : quad_sum(o0 + o1);
+                const float o = LPC == 16 ? hex_sum(o0 + o1) : (LPC == 8 ? oct_sum(o0 + o1) : quad_sum(o0 + o1));
                 if (live && rg == 0) P.out[(size_t)(sd.row0 + t0 + tt) * P.ldo + (size_t)h * P.dv + j] = o;
             }
         }
@@ -767,8 +768,9 @@ int ifa_state_scan_chan_f32(const void *q_f32, size_t ldq, const void *k_f32, si
     P.seqs = (const SeqDesc *)seqs_dev; P.slot_base = (float *const *)slot_base_dev; P.state_off = state_off;
     P.out = (float *)out_f32; P.ldo = ldo;
     const dim3 grid16((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 16)), grid8((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 8));
+    const dim3 grid4((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 4));
 #define IFA_CSCAN(DKV, L, G) if (dk == DKV) { hipLaunchKernelGGL((k_state_scan_chan_reg<DKV, L>), G, dim3(64), 0, ifa_s(stream), P); IFA_LAUNCH_CHECK(); return IFA_OK; }
-    IFA_CSCAN(16, 4, grid16) IFA_CSCAN(32, 4, grid16) IFA_CSCAN(48, 4, grid16) IFA_CSCAN(64, 8, grid8) IFA_CSCAN(96, 8, grid8) IFA_CSCAN(128, 8, grid8)
+    IFA_CSCAN(16, 4, grid16) IFA_CSCAN(32, 4, grid16) IFA_CSCAN(48, 4, grid16) IFA_CSCAN(64, 8, grid8) IFA_CSCAN(96, 8, grid8) IFA_CSCAN(128, 16, grid4)
 #undef IFA_CSCAN
     const size_t smem = ((size_t)dk * 64 + 5 * (size_t)dk) * 4;
     IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_state_scan_chan, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
