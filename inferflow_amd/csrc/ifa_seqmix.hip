@@ -521,7 +521,9 @@ __global__ void __launch_bounds__(64) k_state_scan_chan_reg(ChanScanArgs P)
 #pragma unroll
         for (int x = 0; x < PER; x++) {
             const int e = lane + 64 * x, tt = e / DK, i = e % DK;
-            qs[buf][tt][i] = qr[x]; ks[buf][tt][i] = kr[x]; ws[buf][tt][i] = wr[x]; us[buf][tt][i] = ur[x]; bs[buf][tt][i] = br[x];
+            // channel i = rg DKQ + e lies at [e / 4][rg][e % 4]: the lanes' 16-byte reads of one step are consecutive pieces (no bank is asked twice)
+            const int pi = ((i % DKQ) / 4) * (LPC * 4) + (i / DKQ) * 4 + (i % 4);
+            qs[buf][tt][pi] = qr[x]; ks[buf][tt][pi] = kr[x]; ws[buf][tt][pi] = wr[x]; us[buf][tt][pi] = ur[x]; bs[buf][tt][pi] = br[x];
         }
 #pragma unroll
         for (int tt = 0; tt < SCAN_TB; tt++) vcur[tt] = vnext[tt];
@@ -532,35 +534,40 @@ __global__ void __launch_bounds__(64) k_state_scan_chan_reg(ChanScanArgs P)
         const bool more = t0 + SCAN_TB < sd.n;
         if (more) request(t0 + SCAN_TB);
         const int cnt = min(SCAN_TB, sd.n - t0);
+        // one token.  What does not depend on the state (k v, -b) is formed ahead; from the column's sum sa to the new state are two dependent operations
+        auto token = [&](int tt) {
+            const float vt = vcur[tt];
+            float kv[DKQ], qq[DKQ], ww[DKQ], uu[DKQ], nb[DKQ];
 #pragma unroll
-        for (int tt = 0; tt < SCAN_TB; tt++) {
-            if (tt < cnt) {
-                const float vt = vcur[tt];
-                float kk[DKQ], qq[DKQ], ww[DKQ], uu[DKQ], bb[DKQ];
-#pragma unroll
-                for (int e4 = 0; e4 < DKQ; e4 += 4) {
-                    const float4 k4 = *reinterpret_cast<const float4 *>(&ks[buf][tt][rg * DKQ + e4]), q4 = *reinterpret_cast<const float4 *>(&qs[buf][tt][rg * DKQ + e4]);
-                    const float4 w4 = *reinterpret_cast<const float4 *>(&ws[buf][tt][rg * DKQ + e4]), u4 = *reinterpret_cast<const float4 *>(&us[buf][tt][rg * DKQ + e4]);
-                    const float4 b4 = *reinterpret_cast<const float4 *>(&bs[buf][tt][rg * DKQ + e4]);
-                    kk[e4] = k4.x; kk[e4 + 1] = k4.y; kk[e4 + 2] = k4.z; kk[e4 + 3] = k4.w;
-                    qq[e4] = q4.x; qq[e4 + 1] = q4.y; qq[e4 + 2] = q4.z; qq[e4 + 3] = q4.w;
-                    ww[e4] = w4.x; ww[e4 + 1] = w4.y; ww[e4 + 2] = w4.z; ww[e4 + 3] = w4.w;
-                    uu[e4] = u4.x; uu[e4 + 1] = u4.y; uu[e4 + 2] = u4.z; uu[e4 + 3] = u4.w;
-                    bb[e4] = b4.x; bb[e4 + 1] = b4.y; bb[e4 + 2] = b4.z; bb[e4 + 3] = b4.w;
-                }
-                float r0 = 0.0f, r1 = 0.0f;
-#pragma unroll
-                for (int e = 0; e < DKQ; e += 2) { r0 = fmaf(S[e], uu[e], r0); r1 = fmaf(S[e + 1], uu[e + 1], r1); }
-                const float sa = LPC == 16 ? hex_sum(r0 + r1) : (LPC == 8 ? oct_sum(r0 + r1) : quad_sum(r0 + r1));
-                float o0 = 0.0f, o1 = 0.0f;
-#pragma unroll
-                for (int e = 0; e < DKQ; e += 2) {
-                    S[e] = fmaf(kk[e], vt, fmaf(ww[e], S[e], -bb[e] * sa)); o0 = fmaf(S[e], qq[e], o0);
-                    S[e + 1] = fmaf(kk[e + 1], vt, fmaf(ww[e + 1], S[e + 1], -bb[e + 1] * sa)); o1 = fmaf(S[e + 1], qq[e + 1], o1);
-                }
-                const float o = LPC == 16 ? hex_sum(o0 + o1) : (LPC == 8 ? oct_sum(o0 + o1) : quad_sum(o0 + o1));
-                if (live && rg == 0) P.out[(size_t)(sd.row0 + t0 + tt) * P.ldo + (size_t)h * P.dv + j] = o;
+            for (int e4 = 0; e4 < DKQ; e4 += 4) {
+                const float4 k4 = *reinterpret_cast<const float4 *>(&ks[buf][tt][e4 * LPC + rg * 4]), q4 = *reinterpret_cast<const float4 *>(&qs[buf][tt][e4 * LPC + rg * 4]);
+                const float4 w4 = *reinterpret_cast<const float4 *>(&ws[buf][tt][e4 * LPC + rg * 4]), u4 = *reinterpret_cast<const float4 *>(&us[buf][tt][e4 * LPC + rg * 4]);
+                const float4 b4 = *reinterpret_cast<const float4 *>(&bs[buf][tt][e4 * LPC + rg * 4]);
+                kv[e4] = k4.x * vt; kv[e4 + 1] = k4.y * vt; kv[e4 + 2] = k4.z * vt; kv[e4 + 3] = k4.w * vt;
+                qq[e4] = q4.x; qq[e4 + 1] = q4.y; qq[e4 + 2] = q4.z; qq[e4 + 3] = q4.w;
+                ww[e4] = w4.x; ww[e4 + 1] = w4.y; ww[e4 + 2] = w4.z; ww[e4 + 3] = w4.w;
+                uu[e4] = u4.x; uu[e4 + 1] = u4.y; uu[e4 + 2] = u4.z; uu[e4 + 3] = u4.w;
+                nb[e4] = -b4.x; nb[e4 + 1] = -b4.y; nb[e4 + 2] = -b4.z; nb[e4 + 3] = -b4.w;
             }
+            float r0 = 0.0f, r1 = 0.0f;
+#pragma unroll
+            for (int e = 0; e < DKQ; e += 2) { r0 = fmaf(S[e], uu[e], r0); r1 = fmaf(S[e + 1], uu[e + 1], r1); }
+            const float sa = LPC == 16 ? hex_sum(r0 + r1) : (LPC == 8 ? oct_sum(r0 + r1) : quad_sum(r0 + r1));
+            float o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+            for (int e = 0; e < DKQ; e += 2) {
+                S[e] = fmaf(ww[e], S[e], fmaf(nb[e], sa, kv[e])); o0 = fmaf(S[e], qq[e], o0);
+                S[e + 1] = fmaf(ww[e + 1], S[e + 1], fmaf(nb[e + 1], sa, kv[e + 1])); o1 = fmaf(S[e + 1], qq[e + 1], o1);
+            }
+            const float o = LPC == 16 ? hex_sum(o0 + o1) : (LPC == 8 ? oct_sum(o0 + o1) : quad_sum(o0 + o1));
+            if (live && rg == 0) P.out[(size_t)(sd.row0 + t0 + tt) * P.ldo + (size_t)h * P.dv + j] = o;
+        };
+        if (cnt == SCAN_TB) {      // a whole group: straight-line code, so that a token's read-out overlaps the next token's chain
+#pragma unroll
+            for (int tt = 0; tt < SCAN_TB; tt++) token(tt);
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < SCAN_TB; tt++) if (tt < cnt) token(tt);
         }
         if (more) publish(buf ^ 1);
         __syncthreads();
