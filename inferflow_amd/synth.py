@@ -261,9 +261,9 @@ def bogupel_config(width=2048, vocab=32000, heads=16, kv_heads=4, dim=128, vdim=
     moe = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}
     att = {"type": "attention", "mlp": moe,
            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": float(dim ** -0.5), "mask": {"size": window},
-                     "rot": {"base": 10000.0, "dims": rot_dims, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+                     "rot": {"base": 10000.0, "dims": rot_dims, "scaling": {"factor": 32.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
     dlt = {"type": "general_delta", "mlp": moe, "mixer": {"heads": delta_heads, "dim": delta_dim}, "_rank": rank}
-    return {"architecture": "Bogupel", "width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "logit_scale": 0.5, "loop": {"start": 2, "stop": 4, "times": 2},
+    return {"architecture": "Bogupel", "width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "logit_scale": 0.25, "loop": {"start": 2, "stop": 4, "times": 2},
             "embedding": {"scale": 4.0, "bigram": {"buckets": 65521, "mul_prev": 31337, "mul_cur": 7919}}, "layers": [att, dlt, att, dlt, att, att]}
 
 

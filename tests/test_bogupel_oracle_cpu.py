@@ -19,20 +19,22 @@ def test_dynamic_tanh_at_its_ends():
 
 
 def test_scaled_frequencies_keep_short_waves_and_slow_long_ones():
-    sc = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 64}
+    sc = {"factor": 6.0, "low": 1.5, "high": 5.0, "original": 64}
     plain, scaled = orc.frequencies(10000.0, 32), orc.frequencies(10000.0, 32, sc)
     wl = 2 * math.pi / plain
-    short, long_ = wl < 64 / 4.0, wl > 64 / 1.0
+    short, long_ = wl < 64 / 5.0, wl > 64 / 1.5
     assert short.any() and long_.any() and (~short & ~long_).any()
-    assert np.array_equal(scaled[short], plain[short]) and np.allclose(scaled[long_], plain[long_] / 8.0)
+    assert np.array_equal(scaled[short], plain[short]) and np.allclose(scaled[long_], plain[long_] / 6.0)
     mid = ~short & ~long_
-    assert np.all(scaled[mid] < plain[mid]) and np.all(scaled[mid] > plain[mid] / 8.0)
-    # continuous at both ends of the blend
-    for edge in (64 / 4.0, 64 / 1.0):
+    assert np.all(scaled[mid] < plain[mid]) and np.all(scaled[mid] > plain[mid] / 6.0)
+    # continuous at both ends of the blend: a frequency just on either side of an edge is scaled alike (dims 4, i = 1: f = base^(-1/2))
+    for edge in (64 / 5.0, 64 / 1.5):
         f = 2 * math.pi / edge
-        lo = orc.frequencies(1.0 / (f * (1 - 1e-9)), 4)[1:], orc.frequencies(1.0 / (f * (1 - 1e-9)), 4, sc)[1:]
-        hi = orc.frequencies(1.0 / (f * (1 + 1e-9)), 4)[1:], orc.frequencies(1.0 / (f * (1 + 1e-9)), 4, sc)[1:]
-        assert abs(lo[1] / lo[0] - hi[1] / hi[0]) < 1e-6
+        ratios = []
+        for eps_ in (-1e-9, 1e-9):
+            base = (f * (1 + eps_)) ** -2.0
+            ratios.append(orc.frequencies(base, 4, sc)[1] / orc.frequencies(base, 4)[1])
+        assert abs(ratios[0] - ratios[1]) < 1e-6 and (abs(ratios[0] - 1.0) < 1e-6 or abs(ratios[0] - 1 / 6.0) < 1e-6)
 
 
 def test_rotation_depends_on_distance_only_and_turned_values_come_back():

@@ -179,7 +179,7 @@ def test_values_as_projected_when_neither_normed_nor_turned():
         assert np.abs(got - want).max() < 2e-6 * np.abs(want).max(), (norm, rot)
 
 
-@pytest.mark.parametrize("H,D", [(3, 16), (2, 32), (6, 48), (2, 64), (1, 96), (2, 128), (2, 4), (3, 5), (1, 72), (2, 130)])
+@pytest.mark.parametrize("H,D", [(3, 16), (2, 32), (5, 48), (2, 64), (1, 96), (2, 128), (2, 4), (3, 5), (1, 72), (2, 130)])
 def test_generalized_delta_rule_gates_and_scan(H, D):
     """whole sequences, portions down to one and two tokens, several sequences in a launch, a continued state and a slot that is used again"""
     rng = np.random.default_rng(H * 100 + D)
