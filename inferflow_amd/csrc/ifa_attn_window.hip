@@ -376,14 +376,16 @@ __global__ void __launch_bounds__(256) k_qk_rope_store(float *__restrict__ q, si
     if (do_qk)
     for (int i = tid; i < half; i += blockDim.x) {
         const double a = (double)pos * freq[i];
-        cs[i] = (float)cos(a); cs[half + i] = (float)sin(a);
+        double sn, cn; sincos(a, &sn, &cn);          // (one argument reduction for both)
+        cs[i] = (float)cn; cs[half + i] = (float)sn;
     }
     float *vcs = cs + 2 * half;
     const int vhalf = vdim / 2;
     if (do_v && k && v_freq) {
         for (int i = tid; i < vhalf; i += blockDim.x) {
             const double a = (double)pos * v_freq[i];
-            vcs[i] = (float)cos(a); vcs[vhalf + i] = (float)sin(a);
+            double sn, cn; sincos(a, &sn, &cn);
+            vcs[i] = (float)cn; vcs[vhalf + i] = (float)sn;
         }
     }
     __syncthreads();
@@ -464,7 +466,8 @@ __global__ void __launch_bounds__(256) k_rotate_heads(float *__restrict__ x, siz
     const int pos = sd.pos0 + t - sd.row0;
     for (int i = tid; i < half; i += blockDim.x) {
         const double a = (double)sign * (double)pos * freq[i];
-        cs[i] = (float)cos(a); cs[half + i] = (float)sin(a);
+        double sn, cn; sincos(a, &sn, &cn);          // (one argument reduction for both)
+        cs[i] = (float)cn; cs[half + i] = (float)sn;
     }
     __syncthreads();
     float *xr = x + (size_t)t * ldx;

@@ -100,6 +100,7 @@ struct LayeredNet {
     int opt_fuse_rows = 0;
     int opt_fuse_post = 1;                 // POSTNORM layers, steps of at most 8 rows: norm-add, depth average, next input convolution and its tail in one launch
                                            // SANDWICH layers, every step size: the norm behind a sub-layer and the norm in front of the next one in one launch
+                                           // PRENORM layers: the start of a looped pass inside the norm's launch; steps of at most 8 rows: the norm inside the router's launch
     float *attn_ws = nullptr; size_t attn_ws_bytes = 0;      // partial results of the windowed attention when a (row, head)'s keys are shared out
     int opt_attn_tile_min = 16;            // steps of at least this many rows run the windowed attention through the tiled kernel
     std::vector<ifa_seq_desc> seqs_host;   // the current step's sequences (the tiled attention's grid is sized from them)
@@ -489,8 +490,11 @@ int run_prenorm_layer(ifa_model *m, LLayer &L, size_t T, int nseq, int pass, boo
     void *const *slots = (void *const *)n->slot_base_dev;
     int rc;
     // (the first layer of a looped pass: x += the embedding output, from the second pass on, + the pass's own vector, in the norm's launch)
-    if (pass_start) rc = ifa_add_dyt_f32(n->x, W, T, W, pass > 0 ? n->x0 : nullptr, W, (const bf16_t *)n->loop_step.data + (size_t)pass * W, L.T(IFA_LT_NORM1_ALPHA).data,
-                                         L.T(IFA_LT_NORM1).data, L.T(IFA_LT_NORM1_B).data, n->h, W, s);
+    const bool fused = n->opt_fuse_post != 0;      // (option fuse_post 0: every element-wise step as a launch of its own)
+    if (pass_start && !fused && (rc = ifa_add_rows_vec_f32(n->x, W, T, W, pass > 0 ? n->x0 : nullptr, W, (const bf16_t *)n->loop_step.data + (size_t)pass * W, s))) return rc;
+    if (pass_start && fused)
+        rc = ifa_add_dyt_f32(n->x, W, T, W, pass > 0 ? n->x0 : nullptr, W, (const bf16_t *)n->loop_step.data + (size_t)pass * W, L.T(IFA_LT_NORM1_ALPHA).data,
+                             L.T(IFA_LT_NORM1).data, L.T(IFA_LT_NORM1_B).data, n->h, W, s);
     else rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM1_ALPHA).data, L.T(IFA_LT_NORM1).data, L.T(IFA_LT_NORM1_B).data, n->h, W, s);
     if (rc) return rc;
     if ((rc = linear(m, L.w_in, NI, W, n->h, W, T, L.b_in, nullptr, 1.0f, 0, n->proj, NI))) return rc;
@@ -532,9 +536,12 @@ int run_prenorm_layer(ifa_model *m, LLayer &L, size_t T, int nseq, int pass, boo
     }
     if (!has_moe(sp)) return IFA_OK;
     const int XA = sp.x_experts;
-    if (T <= 8 && XA <= 512) {      // a few rows: the norm and the router's product inside the choice's launch
+    if (T <= 8 && XA <= 512 && fused) {      // a few rows: the norm and the router's product inside the choice's launch
         if ((rc = ifa_moe_dyt_route_rows_f32(sp.x_score, n->x, W, L.T(IFA_LT_NORM2_ALPHA).data, L.T(IFA_LT_NORM2).data, L.T(IFA_LT_NORM2_B).data, n->h, W, T, (int)W,
                                              L.T(IFA_LT_X_ROUTER).data, XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
+    } else if (T <= 8 && XA <= 512) {
+        if ((rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM2_ALPHA).data, L.T(IFA_LT_NORM2).data, L.T(IFA_LT_NORM2_B).data, n->h, W, s))) return rc;
+        if ((rc = ifa_moe_route_rows_scores_f32(sp.x_score, n->h, W, T, (int)W, L.T(IFA_LT_X_ROUTER).data, XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
     } else {
         if ((rc = ifa_dyt_f32(n->x, W, T, W, L.T(IFA_LT_NORM2_ALPHA).data, L.T(IFA_LT_NORM2).data, L.T(IFA_LT_NORM2_B).data, n->h, W, s))) return rc;
         if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_X_ROUTER).data, (size_t)XA, W, n->h, W, T, nullptr, nullptr, 1.0f, 0, n->m2, (size_t)XA))) return rc;

@@ -148,6 +148,20 @@ def test_portions_and_token_by_token_equal_the_whole_prompt(tmp_path, sizes):
     eng.close()
 
 
+def test_folded_launches_and_separate_ops_agree(tmp_path):
+    """the start of a pass inside the norm's launch and the norm inside the router's launch against the same steps as launches of their own"""
+    import inferflow_amd as ia
+    w = fx.random_weights(MIXED, 25)
+    toks = tokens_for(MIXED, 60, 26)
+    want = oracle_logits(MIXED, w, toks)
+    eng = engine_for(tmp_path, MIXED, w)
+    for fuse in (1, 0, 1):
+        ia.check(ia.lib().ifa_model_set_option(eng.worker(), b"fuse_post", fuse))
+        for sizes in ([33, 1], [3, 2], [8, 7, 1]):
+            assert fx.rel_err(run_portions(eng, toks, sizes), want).max() < TOL32, (fuse, sizes)
+    eng.close()
+
+
 @pytest.mark.parametrize("n", [1, 2, 3])
 def test_first_tokens_of_a_sequence(tmp_path, n):
     """the shortest prompts, whole and token by token, on a slot that held a longer sequence before (cache rows, states, last token)"""

@@ -33,7 +33,9 @@ def test_layered_only_library_builds_and_declines_the_standard_network():
     names = ("ifa_model_create_layered", "ifa_model_set_tensor_host", "ifa_model_step_seqs", "ifa_model_logits_f32", "ifa_model_forward",
              "ifa_model_decode", "ifa_model_decode_batch", "ifa_model_kv_slots", "ifa_model_select_kv", "ifa_model_finalize", "ifa_model_destroy",
              "ifa_engine_create_from_dir", "ifa_engine_infer", "ifa_engine_commit", "ifa_engine_last_logits_f32", "ifa_linear_bf16w",
-             "ifa_attention_window_f32", "ifa_state_scan_f32", "ifa_shortconv_silu_f32")
+             "ifa_attention_window_f32", "ifa_state_scan_f32", "ifa_shortconv_silu_f32", "ifa_dyt_f32", "ifa_add_dyt_f32", "ifa_embed_pair_scaled_f32",
+             "ifa_qkv_rope_store_f32", "ifa_rotate_heads_f32", "ifa_attention_kv_sinks_f32", "ifa_chan_delta_gates_f32", "ifa_state_scan_chan_f32",
+             "ifa_moe_dyt_route_rows_f32", "ifa_moe_experts_glu_f32")
     r = subprocess.run([sys.executable, "-c", code, path, ",".join(names)], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr[-2000:]
     assert r.stdout.startswith("[] -4 ") and "standard network" in r.stdout, r.stdout
